@@ -1,9 +1,10 @@
 from .registry import architectures, load_config, register_architecture, resolve
 from .llama import LlamaConfig  # (importing an architecture's module registers it)
-from .spec import (AttentionSpec, LayerCall, ModelSpec, NoPositionSpec, PreNormBlockSpec, RMSNormSpec, RopeSpec,
-                   SwiGLUSpec)
+from .vuzelix import VuzelixConfig
+from .spec import (AttentionSpec, ChannelDeltaSpec, DenseFFSpec, LayerCall, ModelSpec, NoPositionSpec, PreNormBlockSpec, RMSNormSpec,
+                   RopeSpec, StreamBlockSpec, SwiGLUSpec)
 
 __all__ = [
-    "LlamaConfig", "architectures", "load_config", "register_architecture", "resolve", "AttentionSpec", "LayerCall",
+    "LlamaConfig", "VuzelixConfig", "ChannelDeltaSpec", "DenseFFSpec", "StreamBlockSpec", "architectures", "load_config", "register_architecture", "resolve", "AttentionSpec", "LayerCall",
     "ModelSpec", "NoPositionSpec", "PreNormBlockSpec", "RMSNormSpec", "RopeSpec", "SwiGLUSpec",
 ]

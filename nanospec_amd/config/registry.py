@@ -32,6 +32,8 @@ def architectures() -> list[str]:
 def resolve(cfg: dict, generation_cfg: dict | None = None):
     """config.json -> (typed configuration, ModelSpec) of the architecture it names."""
     names = cfg.get("architectures") or []
+    if not names and isinstance(cfg.get("architecture"), str):  # a configuration that names its one architecture as a string
+        names = [cfg["architecture"]]
     name = names[0] if names else _MODEL_TYPES.get(cfg.get("model_type"))
     if name not in _ARCHITECTURES:
         raise ValueError(

@@ -58,6 +58,54 @@ class AttentionSpec:
     position: object  # a position spec (RopeSpec, NoPositionSpec, ...)
     softmax_scale: float  # multiplies q.k before the soft-max
     window: int = 0
+    # Options, each off at its default.  A layer that sets any of them runs the general attention path.
+    value_dim: int = 0  # size of a value head if it is not ``head_dim``
+    qk_norm_eps: float | None = None  # q and k of every head are divided by sqrt(mean(x^2) + eps), no weight, before the scores
+    score_cap: float = 0.0  # > 0: a score s (after the scale) becomes cap * tanh(s / cap)
+    chunk: int = 0  # > 0: a query sees a key only inside its own chunk of this many positions, counted from position 0
+    sink: bool = False  # the soft-max's denominator holds one more term of score 0, which has no value
+    own_kv: bool = True  # False: no key/value projections; the layer reads the cache of the run-order entry it names
+    names: tuple[str, str, str, str] = ("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight")  # after the prefix
+
+    @property
+    def v_dim(self) -> int:
+        return self.value_dim or self.head_dim
+
+    @property
+    def general(self) -> bool:
+        return bool(self.value_dim not in (0, self.head_dim) or self.qk_norm_eps is not None or self.score_cap or self.chunk or self.sink
+                    or not self.own_kv)
+
+
+@dataclass(frozen=True)
+class ChannelDeltaSpec:
+    """The gated delta rule with one decay per head and key channel, behind short causal convolutions of q, k and v.
+    Per head, S [key_dim, value_dim] in 32-bit: S = g_t * S (by key channel); u = beta_t (v_t - S^T k_t); S = S + k_t u^T;
+    o_t = S^T q_t; then o / rms(o) * weight * sigmoid(gate), and the output projection.  The decay's and the gate's
+    projections are products of two matrices whose inner sizes (``decay_rank``, ``gate_rank``) are read from the
+    checkpoint when None; random weights need them given."""
+
+    kind: ClassVar[str] = "channel_delta"
+    hidden: int
+    heads: int
+    kv_heads: int
+    key_dim: int
+    value_dim: int
+    conv: int  # taps of the convolutions, the current token's included
+    norm_eps: float
+    decay_rank: int | None = None
+    gate_rank: int | None = None
+
+
+@dataclass(frozen=True)
+class DenseFFSpec:
+    """down(act(up(x))), dense, no bias.  ``names``: the two matrices after the prefix."""
+
+    kind: ClassVar[str] = "dense"
+    hidden: int
+    intermediate: int
+    activation: str = "gelu_tanh"
+    names: tuple[str, str] = ("up", "down")
 
 
 @dataclass(frozen=True)
@@ -89,6 +137,29 @@ class PreNormBlockSpec:
 
 
 @dataclass(frozen=True)
+class StreamBlockSpec:
+    """A pre-norm block over a residual stream that is kept in 32-bit and may be ``streams`` parallel streams x_1 .. x_S
+    (hyper-connections).  For sublayer q (the mixer, then the feed-forward, which may be None):
+        u = sum_s in_q[s] x_s;  y = sublayer(norm_q(u));  x_t <- sum_s mix_q[s, t] x_s + mult * out_q[t] * y   (all t at once)
+    with the tensors ``prefix + hc_names[q] + "in" | "out" | "mix"``.  ``streams`` = 0: one stream and no such tensors,
+    x <- x + mult * sublayer(norm(x))."""
+
+    kind: ClassVar[str] = "streams"
+    prefix: str
+    mixer_norm: object
+    mixer: object
+    ffn_norm: object | None
+    ffn: object | None
+    streams: int = 0
+    mult: float = 1.0
+    mixer_norm_name: str = "norm1"
+    mixer_prefix: str = "mix."
+    ffn_norm_name: str = "norm2"
+    ffn_prefix: str = "mlp."
+    hc_names: tuple[str, str] = ("hc1.", "hc2.")
+
+
+@dataclass(frozen=True)
 class LayerCall:
     """One entry of the run order.  ``layer`` indexes ``ModelSpec.layers`` (a layer may be named
     by several entries: its weights are used again, each entry with a cache of its own).
@@ -115,6 +186,9 @@ class ModelSpec:
     embed_scale: float = 1.0  # the embedding rows are multiplied by this as they enter the stream
     logit_scale: float = 1.0  # the head's 32-bit logits are multiplied by this ...
     logit_softcap: float = 0.0  # ... and then, if > 0, become softcap * tanh(logit / softcap)
+    # the residual stream between the blocks: 0 = one stream in the model's precision; S >= 1 = S copies in 32-bit, all
+    # equal to the embedding's output at the start and added up before the last norm (blocks of kind "streams")
+    streams: int = 0
 
     def __post_init__(self) -> None:
         for pos, call in enumerate(self.run_order):

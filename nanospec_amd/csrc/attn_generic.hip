@@ -5,8 +5,12 @@
 //
 // Query row i of request b stands at position p = kv_len[b] - q_len[b] + i and sees the keys
 // max(0, p - window + 1) .. p  (window == 0: 0 .. p).          (reference: model/attention.py:22-43)
+// Options that the reference's attention does not have, each off at 0: ``chunk`` (a query also sees no key before the
+// start of its own chunk, floor(p / chunk) * chunk, chunks counted from position 0), ``cap`` (a score s, after the
+// scale, becomes cap * tanh(s / cap)), ``sink`` (the soft-max's denominator holds one more term of score 0 that has no
+// value), and values of another size ``vd`` than the keys' ``hd``.
 // Query head h reads key/value head h / (heads / kv_heads).    (reference: model/attention.py:33)
-// K pages: [page][kv head][token][hd];  V pages: [page][kv head][hd][token].
+// K pages: [page][kv head][token][hd];  V pages: [page][kv head][vd][token].
 #include "common.h"
 
 #define AG_THREADS 256
@@ -15,8 +19,8 @@ template <typename T>
 __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     T* __restrict__ out, const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ token_req, const int* __restrict__ positions,
-    const int* __restrict__ block_table, int table_stride, int heads, int kv_heads, int hd, int page_size, float scale,
-    int window) {
+    const int* __restrict__ block_table, int table_stride, int heads, int kv_heads, int hd, int vd, int page_size, float scale,
+    int window, int chunk, float cap, int sink) {
   extern __shared__ float smem[];  // q_s[hd] | p_s[AG_THREADS] | scratch[16]
   float* q_s = smem;
   float* p_s = smem + hd;
@@ -28,8 +32,10 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
   const T* qrow = q + (size_t)t * q_stride + h * hd;
   for (int d = tid; d < hd; d += AG_THREADS) q_s[d] = to_f(qrow[d]) * scale;
   __syncthreads();
-  const int lo = window > 0 ? max(0, pos - window + 1) : 0;
-  float m = -INFINITY, l = 0.f, acc = 0.f;  // acc: channel `tid` of the output (tid < hd)
+  int lo = window > 0 ? max(0, pos - window + 1) : 0;
+  if (chunk > 0) lo = max(lo, pos / chunk * chunk);
+  const float inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+  float m = -INFINITY, l = 0.f, acc = 0.f;  // acc: channel `tid` of the output (tid < vd)
   for (int c0 = (lo / AG_THREADS) * AG_THREADS; c0 <= pos; c0 += AG_THREADS) {
     const int key = c0 + tid;
     const bool valid = key >= lo && key <= pos;
@@ -39,7 +45,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
       const T* kr = k_cache + (((size_t)page * kv_heads + kvh) * page_size + key % page_size) * hd;
       float dot = 0.f;
       for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], to_f(kr[d]), dot);
-      s = dot;
+      s = cap > 0.f ? cap * tanhf(dot * inv_cap) : dot;
     }
     const float m_new = fmaxf(m, block_max(s, scratch));
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -48,36 +54,93 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     const float alpha = m == -INFINITY ? 0.f : expf(m - m_new);
     l = l * alpha + csum;
     m = m_new;
-    if (tid < hd) {
+    if (tid < vd) {
       acc *= alpha;
       const int hi = min(AG_THREADS, pos - c0 + 1);
       for (int j = max(0, lo - c0); j < hi; ++j) {
         const int kj = c0 + j;
         const int page = table[kj / page_size];
-        const T* vp = v_cache + (((size_t)page * kv_heads + kvh) * hd + tid) * page_size + kj % page_size;
+        const T* vp = v_cache + (((size_t)page * kv_heads + kvh) * vd + tid) * page_size + kj % page_size;
         acc = fmaf(p_s[j], to_f(*vp), acc);
       }
     }
     __syncthreads();
   }
-  if (tid < hd) out[((size_t)t * heads + h) * hd + tid] = from_f<T>(acc / l);
+  if (sink) l += expf(-m);  // the term of score 0, in the units of the running maximum
+  if (tid < vd) out[((size_t)t * heads + h) * vd + tid] = from_f<T>(acc / l);
 }
 
 extern "C" int ns_attn_generic(void* out, const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                const int* token_req, const int* positions, const int* block_table, int table_stride,
-                               int n_tokens, int heads, int kv_heads, int hd, int page_size, float scale, int window,
-                               int dtype, hipStream_t stream) {
-  if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || hd <= 0 || hd > AG_THREADS || page_size <= 0 || window < 0)
+                               int n_tokens, int heads, int kv_heads, int hd, int vd, int page_size, float scale, int window,
+                               int chunk, float cap, int sink, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || hd <= 0 || hd > 1024 || vd <= 0 || vd > AG_THREADS || page_size <= 0 ||
+      window < 0 || chunk < 0 || cap < 0.f)
     return NS_ERR_BAD_ARG;
   if (heads > 65535) return NS_ERR_BAD_ARG;
   dim3 grid(n_tokens, heads);
   const size_t smem = (size_t)(hd + AG_THREADS + 16) * sizeof(float);
   if (dtype == NS_DTYPE_F32)
     attn_generic_kernel<float><<<grid, AG_THREADS, smem, stream>>>((float*)out, (const float*)q, q_stride, (const float*)k_cache,
-        (const float*)v_cache, token_req, positions, block_table, table_stride, heads, kv_heads, hd, page_size, scale, window);
+        (const float*)v_cache, token_req, positions, block_table, table_stride, heads, kv_heads, hd, vd, page_size, scale, window, chunk, cap, sink);
   else if (dtype == NS_DTYPE_BF16)
     attn_generic_kernel<bf16_t><<<grid, AG_THREADS, smem, stream>>>((bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
-        (const bf16_t*)v_cache, token_req, positions, block_table, table_stride, heads, kv_heads, hd, page_size, scale, window);
+        (const bf16_t*)v_cache, token_req, positions, block_table, table_stride, heads, kv_heads, hd, vd, page_size, scale, window, chunk, cap, sink);
+  else
+    return NS_ERR_UNSUPPORTED;
+  return ns_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// What an attention layer without rotation does between its projections and its scores: the queries and keys of every
+// head are divided by their root mean square over the head (``eps`` >= 0; a negative eps leaves them as they are), the
+// queries in place; keys and values go into the pages of their positions.  A row of ``qkv`` is q [heads][hd], then, if
+// the layer has keys and values of its own (``own_kv``), k [kv_heads][hd] and v [kv_heads][vd].
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void unit_kv_write_kernel(T* __restrict__ qkv, int stride, const int* __restrict__ positions, const int* __restrict__ token_req,
+                                     const int* __restrict__ block_table, int table_stride, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                     int heads, int kv_heads, int hd, int vd, int page_size, float eps, int own_kv) {
+  const int t = blockIdx.x, lane = threadIdx.x & (NS_WAVE - 1), wave = threadIdx.x / NS_WAVE, nw = blockDim.x / NS_WAVE;
+  T* row = qkv + (size_t)t * stride;
+  const int pos = positions[t];
+  const int page = own_kv ? block_table[(size_t)token_req[t] * table_stride + pos / page_size] : 0;
+  const int slot = pos % page_size;
+  const int vecs = heads + (own_kv ? kv_heads : 0);
+  for (int vec = wave; vec < vecs; vec += nw) {
+    T* p = row + (size_t)vec * hd;
+    float f = 1.f;
+    if (eps >= 0.f) {
+      float ss = 0.f;
+      for (int d = lane; d < hd; d += NS_WAVE) ss = fmaf(to_f(p[d]), to_f(p[d]), ss);
+      ss = wave_sum(ss);
+      f = 1.f / sqrtf(ss / (float)hd + eps);
+    }
+    if (vec < heads) {
+      if (eps >= 0.f)
+        for (int d = lane; d < hd; d += NS_WAVE) p[d] = from_f<T>(to_f(p[d]) * f);
+    } else {
+      T* dst = k_cache + (((size_t)page * kv_heads + (vec - heads)) * page_size + slot) * hd;
+      for (int d = lane; d < hd; d += NS_WAVE) dst[d] = from_f<T>(to_f(p[d]) * f);
+    }
+  }
+  if (own_kv) {
+    const T* v = row + (size_t)(heads + kv_heads) * hd;
+    for (int i = threadIdx.x; i < kv_heads * vd; i += blockDim.x)
+      v_cache[(((size_t)page * kv_heads + i / vd) * vd + i % vd) * page_size + slot] = v[i];
+  }
+}
+
+extern "C" int ns_unit_kv_write(void* qkv, int stride, const int* positions, const int* token_req, const int* block_table, int table_stride,
+                                void* k_cache, void* v_cache, int n_tokens, int heads, int kv_heads, int hd, int vd, int page_size,
+                                float eps, int own_kv, int dtype, hipStream_t stream) {
+  if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || hd <= 0 || vd <= 0 || page_size <= 0) return NS_ERR_BAD_ARG;
+  if (dtype == NS_DTYPE_F32)
+    unit_kv_write_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)qkv, stride, positions, token_req, block_table, table_stride,
+                                                               (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, vd, page_size, eps, own_kv);
+  else if (dtype == NS_DTYPE_BF16)
+    unit_kv_write_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((bf16_t*)qkv, stride, positions, token_req, block_table, table_stride,
+                                                                (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, vd, page_size, eps, own_kv);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();

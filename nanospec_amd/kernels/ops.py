@@ -644,34 +644,64 @@ def rope_kv_from_partial(p: PartialSums, q_out: torch.Tensor, positions, token_r
 # ------------------------------------------------------------------------------------------------ attention
 
 
-def _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim):
+def _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim, v_dim: int | None = None):
     _gpu(q, out, k_cache, v_cache)
+    v_dim = head_dim if v_dim is None else v_dim
     page = k_cache.shape[2] if k_cache.dim() == 4 else 0
-    if (k_cache.dim() != 4 or k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, head_dim, page)
+    if (k_cache.dim() != 4 or k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, v_dim, page)
             or not k_cache.is_contiguous() or not v_cache.is_contiguous() or k_cache.dtype != q.dtype or v_cache.dtype != q.dtype):
         raise KernelRefused("attention: cache pages do not fit heads, head size or dtype")
     if q.stride(1) != 1 or q.shape[1] < heads * head_dim:
         raise KernelRefused("attention: q rows must hold heads * head_dim contiguous values")
-    if out.shape != (q.shape[0], heads * head_dim) or not out.is_contiguous() or out.dtype != q.dtype:
-        raise KernelRefused("attention: out must be contiguous [tokens, heads * head_dim]")
+    if out.shape != (q.shape[0], heads * v_dim) or not out.is_contiguous() or out.dtype != q.dtype:
+        raise KernelRefused("attention: out must be contiguous [tokens, heads * value size]")
     if heads % kv_heads:
         raise KernelRefused(f"attention: {heads} heads are not a multiple of {kv_heads} key/value heads")
     return page
 
 
 def attention_generic(q, out, k_cache, v_cache, token_req, positions, block_table, heads: int, kv_heads: int, head_dim: int,
-                      scale: float, window: int = 0) -> torch.Tensor:
-    """Attention of every token's query over its request's pages; any head size up to 256, either dtype."""
-    page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim)
+                      scale: float, window: int = 0, v_dim: int | None = None, chunk: int = 0, cap: float = 0.0,
+                      sink: bool = False) -> torch.Tensor:
+    """Attention of every token's query over its request's pages; any key size up to 1024 and value size up to 256, either
+    dtype.  ``chunk`` > 0: a query sees no key before the start of its own chunk of positions; ``cap`` > 0: scores become
+    cap * tanh(score / cap); ``sink``: one more term of score 0 without a value in the soft-max's denominator."""
+    v_dim = head_dim if v_dim is None else v_dim
+    page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim, v_dim)
     _i32(token_req, "token_req"), _i32(positions, "positions"), _i32(block_table, "block_table")
-    if head_dim > 256:
-        raise KernelRefused(f"attention_generic takes head sizes up to 256, not {head_dim}")
+    if head_dim > 1024 or v_dim > 256:
+        raise KernelRefused(f"attention_generic takes key sizes up to 1024 and value sizes up to 256, not {head_dim} and {v_dim}")
     n = q.shape[0]
     _check(build.core().ns_attn_generic(_ptr(out), _ptr(q), c_int(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(token_req),
                                         _ptr(positions), _ptr(block_table), c_int(block_table.stride(0)), c_int(n), c_int(heads),
-                                        c_int(kv_heads), c_int(head_dim), c_int(page), c_float(scale), c_int(window),
-                                        c_int(_dtype_code(q)), _stream()), "attention_generic")
+                                        c_int(kv_heads), c_int(head_dim), c_int(v_dim), c_int(page), c_float(scale), c_int(window),
+                                        c_int(chunk), c_float(cap), c_int(1 if sink else 0), c_int(_dtype_code(q)), _stream()),
+           "attention_generic")
     return out
+
+
+def unit_kv_write(qkv: torch.Tensor, positions, token_req, block_table, k_cache, v_cache, heads: int, kv_heads: int, head_dim: int,
+                  v_dim: int, eps: float | None, own_kv: bool = True) -> None:
+    """For attention without rotation.  A row of ``qkv`` is q [heads, head_dim] and, with ``own_kv``, k [kv_heads, head_dim]
+    and v [kv_heads, v_dim].  With ``eps`` not None every head's q (in place) and k are divided by their root mean square,
+    x / sqrt(mean(x^2) + eps); k and v of every token go into the pages ``block_table[token_req[t], position // page]``:
+    k_cache [pages, kv_heads, page, head_dim], v_cache [pages, kv_heads, v_dim, page]."""
+    _gpu(qkv, positions, token_req, block_table, k_cache, v_cache)
+    n = positions.numel()
+    width = heads * head_dim + (kv_heads * (head_dim + v_dim) if own_kv else 0)
+    if qkv.dim() != 2 or qkv.shape[0] != n or qkv.shape[1] < width or qkv.stride(1) != 1:
+        raise KernelRefused(f"unit_kv_write: qkv must be [{n}, {width}]")
+    _i32(positions, "positions"), _i32(token_req, "token_req"), _i32(block_table, "block_table")
+    if token_req.numel() != n or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelRefused("unit_kv_write: token_req is per token, block_table int32 [requests, pages]")
+    page = k_cache.shape[2] if k_cache.dim() == 4 else 0
+    if (k_cache.dim() != 4 or k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, v_dim, page)
+            or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
+        raise KernelRefused("unit_kv_write: cache pages do not fit heads, sizes or dtype")
+    _check(build.core().ns_unit_kv_write(_ptr(qkv), c_int(qkv.stride(0)), _ptr(positions), _ptr(token_req), _ptr(block_table),
+                                         c_int(block_table.stride(0)), _ptr(k_cache), _ptr(v_cache), c_int(n), c_int(heads), c_int(kv_heads),
+                                         c_int(head_dim), c_int(v_dim), c_int(page), c_float(-1.0 if eps is None else eps),
+                                         c_int(1 if own_kv else 0), c_int(_dtype_code(qkv)), _stream()), "unit_kv_write")
 
 
 def mfma_attention_takes(dtype, head_dim: int, page_size: int) -> bool:
@@ -729,6 +759,163 @@ def attention_prompt_form(head_dim: int, page_size: int) -> int:
     on the 32x32 matrix instruction with loads straight into LDS, 16 the one on the 16x16 instruction with keys shared
     through LDS, 0 the one without sharing."""
     return int(build.attn(head_dim, page_size).ns_attn_prompt_form())
+
+
+# ------------------------------------------------------------------------------------------------ 32-bit streams
+
+MAX_STREAMS = 16
+ACTIVATIONS = {"gelu_tanh": 0, "silu": 1}
+
+
+def _f32(t: torch.Tensor, name: str) -> torch.Tensor:
+    if t.dtype != torch.float32 or not t.is_contiguous() or not t.is_cuda:
+        raise KernelRefused(f"{name} must be a contiguous float32 tensor on the GPU")
+    return t
+
+
+def embed_streams(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """out[i, s, :] = table[ids[i]] * scale for every copy s of the stream; ``out`` float32 [tokens, copies, hidden]."""
+    _gpu(table, ids)
+    _i32(ids, "ids"), _f32(out, "out")
+    n, hidden = ids.numel(), table.shape[1]
+    if out.dim() != 3 or out.shape[0] != n or out.shape[2] != hidden or not 1 <= out.shape[1] <= MAX_STREAMS or not table.is_contiguous():
+        raise KernelRefused(f"embed_streams: out must be float32 [{n}, copies <= {MAX_STREAMS}, {hidden}]")
+    _check(build.core().ns_embed_streams(_ptr(out), _ptr(table), _ptr(ids), c_int(n), c_int(hidden), c_int(out.shape[1]), c_float(scale),
+                                         c_int(_dtype_code(table)), _stream()), "embed_streams")
+    return out
+
+
+def stream_read_norm(x: torch.Tensor, coeff: torch.Tensor, weight: torch.Tensor, eps: float, rows: torch.Tensor | None = None,
+                     out: torch.Tensor | None = None, sum_out: torch.Tensor | None = None) -> torch.Tensor:
+    """u = sum_s coeff[s] x[r, s, :] with r = rows[i] (or i); out[i] = weight * u / sqrt(mean(u^2) + eps) in the weight's dtype.
+    ``x`` float32 [tokens, S, W]; ``sum_out`` (float32 [n, W], optional) also receives u."""
+    _f32(x, "x"), _f32(coeff, "coeff")
+    _gpu(weight, rows, out, sum_out)
+    if x.dim() != 3 or coeff.numel() != x.shape[1] or x.shape[1] > MAX_STREAMS or weight.shape != (x.shape[2],) or not weight.is_contiguous():
+        raise KernelRefused("stream_read_norm: x is [tokens, S, W], coeff [S], weight [W]")
+    if rows is not None:
+        _i32(rows, "rows")
+    n = rows.numel() if rows is not None else x.shape[0]
+    S, W = x.shape[1], x.shape[2]
+    if out is None:
+        out = torch.empty((n, W), dtype=weight.dtype, device=x.device)
+    if out.shape != (n, W) or out.dtype != weight.dtype or not out.is_contiguous():
+        raise KernelRefused("stream_read_norm: out must be contiguous [rows, W] of the weight's dtype")
+    if sum_out is not None and (_f32(sum_out, "sum_out").shape != (n, W)):
+        raise KernelRefused("stream_read_norm: sum_out must be float32 [rows, W]")
+    _check(build.core().ns_stream_read_norm(_ptr(out), _ptr(sum_out), _ptr(x), _ptr(coeff), _ptr(weight), _ptr(rows), c_int(n), c_int(S),
+                                            c_int(W), c_float(eps), c_int(_dtype_code(weight)), _stream()), "stream_read_norm")
+    return out
+
+
+def stream_write(x: torch.Tensor, mix: torch.Tensor, gain: torch.Tensor, y: torch.Tensor) -> None:
+    """In place, all streams at once from the old ones: x[r, t, :] = sum_s mix[s, t] x[r, s, :] + gain[t] * y[r, :]."""
+    _f32(x, "x"), _f32(mix, "mix"), _f32(gain, "gain")
+    _gpu(y)
+    if x.dim() != 3 or mix.shape != (x.shape[1], x.shape[1]) or gain.shape != (x.shape[1],) or x.shape[1] > MAX_STREAMS:
+        raise KernelRefused("stream_write: x is [tokens, S, W], mix [S, S] (from, to), gain [S]")
+    if y.dim() != 2 or y.shape != (x.shape[0], x.shape[2]) or y.stride(1) != 1:
+        raise KernelRefused("stream_write: y must be [tokens, W]")
+    _check(build.core().ns_stream_write(_ptr(x), _ptr(mix), _ptr(gain), _ptr(y), c_int(y.stride(0)), c_int(x.shape[0]), c_int(x.shape[1]),
+                                        c_int(x.shape[2]), c_int(_dtype_code(y)), _stream()), "stream_write")
+
+
+def activation(x: torch.Tensor, kind: str, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out = act(x) element by element (in place by default); ``kind`` one of ``ACTIVATIONS``."""
+    _gpu(x, out)
+    if kind not in ACTIVATIONS:
+        raise KernelRefused(f"activation {kind!r} is not known (known: {sorted(ACTIVATIONS)})")
+    out = x if out is None else out
+    if not x.is_contiguous() or not out.is_contiguous() or out.shape != x.shape or out.dtype != x.dtype:
+        raise KernelRefused("activation: x and out must be contiguous and alike")
+    _check(build.core().ns_activation(_ptr(out), _ptr(x), c_size_t(x.numel()), c_int(ACTIVATIONS[kind]), c_int(_dtype_code(x)), _stream()),
+           "activation")
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ delta rule
+
+MAX_CONV_TAPS = 16
+DELTA_MAX_KEY_DIM = 1024
+
+
+def _state_args(state: torch.Tensor, what: str):
+    if state.dtype != torch.float32 or state.dim() != 2 or not state.is_contiguous() or not state.is_cuda:
+        raise KernelRefused(f"{what}: the state is float32 [slots, floats per slot] on the GPU")
+    return _ptr(state), c_size_t(state.shape[1])
+
+
+def conv_silu_carry(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, conv_off: int, token_req, qo_indptr, state_slots,
+                    out: torch.Tensor) -> torch.Tensor:
+    """A short causal convolution over time per channel, then SiLU, across steps.  ``x`` [tokens, >= C] (its first C columns
+    are convolved), ``taps`` float32 [C, K] whose last column multiplies the current token; the K - 1 inputs before a
+    request's first token of this step are read from ``state[slot, conv_off:]`` as [K - 1, C] (zeros for a new request)
+    and replaced afterwards by the last K - 1 inputs including this step's.  ``out`` float32 [tokens, C]."""
+    _gpu(x), _f32(taps, "taps"), _f32(out, "out")
+    for name, t in (("token_req", token_req), ("qo_indptr", qo_indptr), ("state_slots", state_slots)):
+        _i32(t, name)
+    C, K = taps.shape
+    n, reqs = token_req.numel(), state_slots.numel()
+    if x.dim() != 2 or x.shape[0] != n or x.shape[1] < C or x.stride(1) != 1 or out.shape != (n, C) or qo_indptr.numel() != reqs + 1:
+        raise KernelRefused("conv_silu_carry: x is [tokens, >= C], out float32 [tokens, C], qo_indptr [requests + 1]")
+    if K > MAX_CONV_TAPS or conv_off + (K - 1) * C > state.shape[1]:
+        raise KernelRefused(f"conv_silu_carry: at most {MAX_CONV_TAPS} taps, and the carried inputs must fit the slot")
+    sp, stride = _state_args(state, "conv_silu_carry")
+    _check(build.core().ns_conv_silu_carry(_ptr(out), _ptr(x), c_int(x.stride(0)), _ptr(taps), sp, stride, c_size_t(conv_off), _ptr(token_req),
+                                           _ptr(qo_indptr), _ptr(state_slots), c_int(n), c_int(reqs), c_int(C), c_int(K),
+                                           c_int(_dtype_code(x)), _stream()), "conv_silu_carry")
+    return out
+
+
+def delta_prep(qkv: torch.Tensor, a: torch.Tensor, b: torch.Tensor, dt_bias: torch.Tensor, a_log: torch.Tensor, heads: int, kv_heads: int,
+               key_dim: int, g: torch.Tensor, beta: torch.Tensor) -> None:
+    """What the delta rule's recurrence reads, in 32-bit.  In place in ``qkv`` (float32 [tokens, C], q [kv_heads, key_dim]
+    then k alike then v): q and k of every head become x / sqrt(sum(x^2) + 1e-6), q times key_dim^(-1/2).
+    g[t, h, d] = exp(-exp(a_log[h]) * softplus(a[t, h, d] + dt_bias[h, d])); beta[t, h] = sigmoid(b[t, h]).
+    ``a`` [tokens, >= heads * key_dim] and ``b`` [tokens, >= heads] may be column slices of wider tensors."""
+    _f32(qkv, "qkv"), _f32(g, "g"), _f32(beta, "beta"), _f32(dt_bias, "dt_bias"), _f32(a_log, "a_log")
+    _gpu(a, b)
+    n = qkv.shape[0]
+    if (qkv.dim() != 2 or qkv.shape[1] < 2 * kv_heads * key_dim or a.dtype != b.dtype or a.stride(1) != 1 or b.stride(1) != 1
+            or a.shape[0] != n or b.shape[0] != n or a.shape[1] < heads * key_dim or b.shape[1] < heads or g.shape != (n, heads * key_dim)
+            or beta.shape != (n, heads) or dt_bias.numel() != heads * key_dim or a_log.numel() != heads or heads % kv_heads):
+        raise KernelRefused("delta_prep: operands do not fit heads and key size")
+    _check(build.core().ns_delta_prep(_ptr(qkv), c_int(qkv.shape[1]), _ptr(g), _ptr(beta), _ptr(a), c_int(a.stride(0)), _ptr(b),
+                                      c_int(b.stride(0)), _ptr(dt_bias), _ptr(a_log), c_int(n), c_int(heads), c_int(kv_heads), c_int(key_dim),
+                                      c_int(_dtype_code(a)), _stream()), "delta_prep")
+
+
+def delta_scan(qkv: torch.Tensor, g: torch.Tensor, beta: torch.Tensor, state: torch.Tensor, qo_indptr, state_slots, heads: int,
+               kv_heads: int, key_dim: int, value_dim: int, out: torch.Tensor) -> torch.Tensor:
+    """The gated delta rule over every request's tokens of this step, from and into ``state[slot, : heads * key_dim *
+    value_dim]`` (S [heads, key_dim, value_dim] per request): S = g_t * S (by key channel); u = beta_t (v_t - S^T k_t);
+    S = S + k_t u^T; o_t = S^T q_t.  ``qkv`` as ``delta_prep`` leaves it; ``out`` float32 [tokens, heads * value_dim]."""
+    _f32(qkv, "qkv"), _f32(g, "g"), _f32(beta, "beta"), _f32(out, "out")
+    _i32(qo_indptr, "qo_indptr"), _i32(state_slots, "state_slots")
+    n, reqs = qkv.shape[0], state_slots.numel()
+    C = 2 * kv_heads * key_dim + heads * value_dim
+    if (qkv.shape != (n, C) or g.shape != (n, heads * key_dim) or beta.shape != (n, heads) or out.shape != (n, heads * value_dim)
+            or qo_indptr.numel() != reqs + 1 or heads % kv_heads or key_dim > DELTA_MAX_KEY_DIM
+            or state.shape[1] < heads * key_dim * value_dim):
+        raise KernelRefused("delta_scan: operands do not fit heads, key size and value size")
+    sp, stride = _state_args(state, "delta_scan")
+    _check(build.core().ns_delta_scan(_ptr(out), _ptr(qkv), c_int(C), _ptr(g), _ptr(beta), sp, stride, _ptr(qo_indptr), _ptr(state_slots),
+                                      c_int(reqs), c_int(heads), c_int(kv_heads), c_int(key_dim), c_int(value_dim), _stream()), "delta_scan")
+    return out
+
+
+def gated_rms(o: torch.Tensor, gate: torch.Tensor, weight: torch.Tensor, eps: float, heads: int, out: torch.Tensor) -> torch.Tensor:
+    """out[t, h, :] = o[t, h, :] / sqrt(mean(o[t, h, :]^2) + eps) * weight * sigmoid(gate[t, h, :]); ``o`` float32 [tokens,
+    heads * E], ``weight`` float32 [E], ``gate`` (may be a column slice) and ``out`` in the model's dtype."""
+    _f32(o, "o"), _f32(weight, "weight")
+    _gpu(gate, out)
+    n, width = o.shape
+    if (width % heads or weight.numel() != width // heads or gate.shape[0] != n or gate.shape[1] < width or gate.stride(1) != 1
+            or out.shape != (n, width) or not out.is_contiguous() or out.dtype != gate.dtype):
+        raise KernelRefused("gated_rms: operands do not fit heads and value size")
+    _check(build.core().ns_gated_rms(_ptr(out), _ptr(o), _ptr(gate), c_int(gate.stride(0)), _ptr(weight), c_int(n), c_int(heads),
+                                     c_int(width // heads), c_float(eps), c_int(_dtype_code(gate)), _stream()), "gated_rms")
+    return out
 
 
 # ------------------------------------------------------------------------------------------------ sampling

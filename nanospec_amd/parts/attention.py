@@ -150,33 +150,37 @@ class Attention:
     @property
     def _names(self):
         p = self.prefix
-        return p + "q_proj.weight", p + "k_proj.weight", p + "v_proj.weight", p + "o_proj.weight"
+        return tuple(p + name for name in self.spec.names)
 
     def wanted(self) -> dict:
         s = self.spec
         q, k, v, o = self._names
-        return {
-            q: ((s.heads * s.head_dim, s.hidden), "linear"),
-            k: ((s.kv_heads * s.head_dim, s.hidden), "linear"),
-            v: ((s.kv_heads * s.head_dim, s.hidden), "linear"),
-            o: ((s.hidden, s.heads * s.head_dim), "linear"),
-            **self.position.wanted(),
-        }
+        out = {q: ((s.heads * s.head_dim, s.hidden), "linear"), o: ((s.hidden, s.heads * s.v_dim), "linear"), **self.position.wanted()}
+        if s.own_kv:
+            out[k] = ((s.kv_heads * s.head_dim, s.hidden), "linear")
+            out[v] = ((s.kv_heads * s.v_dim, s.hidden), "linear")
+        return out
 
     def load(self, get, dtype, device, layouts: str = "both") -> None:
         s = self.spec
         plain = layouts == "both"
         q, k, v, o = self._names
-        rows = (s.heads + 2 * s.kv_heads) * s.head_dim
+        rows = s.heads * s.head_dim + (s.kv_heads * (s.head_dim + s.v_dim) if s.own_kv else 0)
         wqkv = torch.empty((rows, s.hidden), dtype=dtype, device=device)
         at = 0
-        for name in (q, k, v):
+        for name in (q, k, v) if s.own_kv else (q,):
             t = get(name)
             wqkv[at : at + t.shape[0]].copy_(t)
             at += t.shape[0]
         self.position.load(get, dtype, device)
         # how the position encoding pairs channels and scales cosine and sine (the kernels' ``RopeForm``)
         self._form = dict(interleaved=bool(getattr(self.position, "interleaved", False)), factor=float(getattr(self.position, "factor", 1.0)))
+        if s.general:
+            # the general path: one product for what the layer projects, then norm / cache write and attention as kernels
+            self.wqkv_rope = None
+            self.wqkv = LinearWeight(wqkv, keep_plain=plain)
+            self.wo = LinearWeight(get(o).to(device=device, dtype=dtype).contiguous(), keep_plain=plain)
+            return
         # for few rows the stacked matrix is streamed by a kernel that rotates and writes the cache in its epilogue; it
         # wants the rows tiled in an order of its own
         rot = self.position.rotary_dim
@@ -188,7 +192,10 @@ class Attention:
         self.wo = LinearWeight(get(o).to(device=device, dtype=dtype).contiguous(), keep_plain=plain)
 
     def cache_need(self):
-        return PagedNeed(self.spec.kv_heads, self.spec.head_dim, self.spec.window)
+        s = self.spec
+        if not s.own_kv:
+            return None  # it reads the cache of the run-order entry that its LayerCall names
+        return PagedNeed(s.kv_heads, s.head_dim, s.window, 0 if s.v_dim == s.head_dim else s.v_dim)
 
     def batch_plans(self) -> list:
         """What this mixer asks the batch builder to put on the device each step (``engine.context``)."""
@@ -199,6 +206,8 @@ class Attention:
 
     def links_norms(self, rows: int) -> bool:
         """Whether, for this many rows, ``forward`` takes a ``PreNormed`` input and an ``IntoResidual`` ending."""
+        if self.spec.general:
+            return False
         first = self.wqkv_rope is not None or self.wqkv.links_norms(rows)
         return rows <= 16 and first and self.wo.links_norms(rows)
 
@@ -210,6 +219,8 @@ class Attention:
             raise ValueError(f"position {ctx.max_position} is beyond the model's {pos.max_positions} positions")
         qkv = ctx.arena.take((n, self.wqkv.n), x.dtype)
         table = ctx.block_tables[cache.group]
+        if s.general:
+            return self._forward_general(ctx, x, cache, owns_cache, out, residual, qkv, table)
         if self.wqkv_rope is not None and n <= 16 and ops.tiled_takes(x.x if isinstance(x, ops.PreNormed) else x, s.hidden):
             ops.linear_qkv_rope(x, self.wqkv_rope, qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v,
                                 s.heads, s.kv_heads, s.head_dim, pos.rotary_dim, write_kv=owns_cache, **self._form)
@@ -238,6 +249,33 @@ class Attention:
         else:
             ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads,
                                   s.head_dim, s.softmax_scale, window=s.window)
+        if residual is not None:
+            return self.wo.into_residual(att, residual, arena=ctx.arena, plain_copy=not ctx.captured)
+        return self.wo(att, out=out, arena=ctx.arena, plain_copy=not ctx.captured)
+
+
+    def _forward_general(self, ctx, x, cache, owns_cache, out, residual, qkv, table):
+        """Attention with any of the spec's options: values of another size than the keys, unit-RMS queries and keys, capped
+        scores, a chunked mask, a sink, keys and values of another layer.  The cache holds keys as the scores meet them
+        (after norm and rotation), so a layer that borrows them brings only its queries."""
+        s, pos = self.spec, self.position
+        n = x.shape[0]
+        if s.own_kv != bool(owns_cache):
+            raise ValueError("an attention layer writes the cache exactly if it has key/value projections of its own")
+        if cache.k.shape[1:] != (s.kv_heads, cache.k.shape[2], s.head_dim) or cache.v.shape[2] != s.v_dim:
+            raise ValueError("the cache that this layer reads has other heads or sizes than the layer")
+        self.wqkv(x, out=qkv, arena=ctx.arena, plain_copy=not ctx.captured)
+        if pos.rotary_dim:
+            if s.qk_norm_eps is not None or s.v_dim != s.head_dim or not s.own_kv:
+                raise ops.KernelRefused("rotation together with unit-RMS queries and keys, another value size or borrowed keys is not built")
+            ops.rope_kv_write(qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v, s.heads, s.kv_heads,
+                              s.head_dim, pos.rotary_dim, write_kv=True, **self._form)
+        else:
+            ops.unit_kv_write(qkv, ctx.positions, ctx.token_req, table, cache.k, cache.v, s.heads, s.kv_heads, s.head_dim, s.v_dim,
+                              s.qk_norm_eps, own_kv=s.own_kv)
+        att = ctx.arena.take((n, s.heads * s.v_dim), x.dtype)
+        ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads, s.head_dim,
+                              s.softmax_scale, window=s.window, v_dim=s.v_dim, chunk=s.chunk, cap=s.score_cap, sink=s.sink)
         if residual is not None:
             return self.wo.into_residual(att, residual, arena=ctx.arena, plain_copy=not ctx.captured)
         return self.wo(att, out=out, arena=ctx.arena, plain_copy=not ctx.captured)

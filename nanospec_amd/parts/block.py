@@ -105,3 +105,104 @@ class PreNormBlock:
 
 
 registry.register("block", "prenorm", PreNormBlock)
+
+
+class StreamBlock:
+    """A pre-norm block over a 32-bit residual stream of S parallel copies x [tokens, S, width] (hyper-connections; S = 1
+    without mixing tensors is the plain residual with its sum in 32-bit).  For each sublayer (mixer, then feed-forward
+    if there is one):
+        u = sum_s in[s] x_s;  y = sublayer(norm(u));  x_t <- sum_s mix[s, t] x_s + mult * out[t] * y   for all t at once
+    The read is one kernel with the norm (``norm.read_streams``), the write another; sublayers compute in the model's
+    precision and never see the streams."""
+
+    stream_form = "streams"  # what ``forward`` takes as ``resid``: float32 [tokens, S, width], updated in place
+
+    def __init__(self, spec, prefix: str | None = None) -> None:
+        p = spec.prefix if prefix is None else prefix
+        self.spec, self.prefix = spec, p
+        self.copies = max(1, spec.streams)
+        self.mixer_norm = registry.build("norm", spec.mixer_norm, p + spec.mixer_norm_name)
+        self.mixer = registry.build("mixer", spec.mixer, p + spec.mixer_prefix)
+        self.ffn = registry.build("ffn", spec.ffn, p + spec.ffn_prefix) if spec.ffn is not None else None
+        self.ffn_norm = registry.build("norm", spec.ffn_norm, p + spec.ffn_norm_name) if spec.ffn is not None else None
+        self.parts = tuple(x for x in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if x is not None)
+        for norm in (self.mixer_norm, self.ffn_norm):
+            if norm is not None and not hasattr(norm, "read_streams"):
+                raise ValueError(f"a norm of kind {norm.spec.kind!r} cannot read a 32-bit stream (it has no read_streams)")
+        self._hc: list = []  # per sublayer: (in [S], mix [S, S], mult * out [S]) float32 on the device
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(getattr(p, "graph_safe", False) for p in self.parts)
+
+    def _hc_names(self):
+        return [self.prefix + q + t for q in self.spec.hc_names[: 2 if self.ffn is not None else 1] for t in ("in", "out", "mix")]
+
+    def wanted(self) -> dict:
+        out = {}
+        for p in self.parts:
+            out.update(p.wanted())
+        if self.spec.streams:
+            S = self.copies
+            # laws under which random streams neither die out nor blow up: read about the mean, write about evenly,
+            # mix close to the identity
+            law = lambda mean, std: (lambda shape, gen: mean + std * torch.randn(shape, generator=gen, dtype=torch.float32, device=gen.device))
+            for name in self._hc_names():
+                if name.endswith("mix"):
+                    out[name] = ((S, S), lambda shape, gen: torch.eye(S, device=gen.device) * 0.9 + 0.1 / S
+                                 + 0.05 * torch.randn(shape, generator=gen, dtype=torch.float32, device=gen.device))
+                else:
+                    out[name] = ((S,), law(1.0 / S if name.endswith("in") else 1.0, 0.1))
+        return out
+
+    takes_layouts = True
+
+    def load(self, get, dtype, device, layouts: str = "both") -> None:
+        for p in self.parts:
+            if getattr(p, "takes_layouts", False):
+                p.load(get, dtype, device, layouts)
+            else:
+                p.load(get, dtype, device)
+        S, m = self.copies, float(self.spec.mult)
+        self._hc = []
+        f32 = lambda t: t.to(device=device, dtype=torch.float32).contiguous()
+        for q in range(2 if self.ffn is not None else 1):
+            if self.spec.streams:
+                pre = self.prefix + self.spec.hc_names[q]
+                self._hc.append((f32(get(pre + "in")), f32(get(pre + "mix")), f32(get(pre + "out")) * m))
+            else:
+                self._hc.append((torch.ones(1, device=device), torch.ones((1, 1), device=device), torch.full((1,), m, device=device)))
+
+    def cache_need(self):
+        return self.mixer.cache_need()
+
+    def batch_plans(self) -> list:
+        return [plan for p in self.parts for plan in getattr(p, "batch_plans", list)()]
+
+    def max_positions(self) -> int | None:
+        limits = [p.max_positions() for p in self.parts if hasattr(p, "max_positions")]
+        limits = [n for n in limits if n is not None]
+        return min(limits) if limits else None
+
+    def forward(self, ctx, resid, delta, cache, owns_cache, delta_out):
+        """``resid``: float32 [tokens, S, width], updated in place; ``delta`` and ``delta_out`` are not used (nothing is
+        ever left to be added)."""
+        n, S, W = resid.shape
+        if S != self.copies:
+            raise ValueError(f"the block is built for {self.copies} streams, the model carries {S}")
+        mark = ctx.arena.mark()
+        dtype = self.mixer_norm.weight.dtype
+        a, mix, gain = self._hc[0]
+        h = self.mixer_norm.read_streams(ctx, resid, a, out=ctx.arena.take((n, W), dtype))
+        y = self.mixer.forward(ctx, h, cache, owns_cache, out=ctx.arena.take((n, W), dtype))
+        ops.stream_write(resid, mix, gain, y)
+        if self.ffn is not None:
+            a, mix, gain = self._hc[1]
+            h = self.ffn_norm.read_streams(ctx, resid, a, out=h)
+            y = self.ffn.forward(ctx, h, out=y)
+            ops.stream_write(resid, mix, gain, y)
+        ctx.arena.release(mark)
+        return None
+
+
+registry.register("block", "streams", StreamBlock)

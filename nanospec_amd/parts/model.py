@@ -41,6 +41,16 @@ class DecoderModel:
         self._max_positions = "?"  # not asked yet
         # what every entry of the run order keeps in the cache
         self.cache_needs = [self.layers[c.layer].cache_need() if c.cache_from is None else None for c in spec.run_order]
+        # the residual stream between the blocks: one tensor in the model's precision, or ``spec.streams`` copies in 32-bit
+        forms = {getattr(layer, "stream_form", "single") for layer in self.layers}
+        if len(forms) > 1 or (forms == {"streams"}) != bool(spec.streams):
+            raise ValueError(f"the blocks carry the residual stream as {sorted(forms)}, the model as {'streams' if spec.streams else 'single'}")
+        if spec.streams and not hasattr(self.final_norm, "read_streams"):
+            raise ValueError("the last norm cannot read a 32-bit stream (it has no read_streams)")
+        self._ones: torch.Tensor | None = None
+        # for tests and debugging: called as layer_probe(run-order entry, float32 [tokens, hidden]) with the sum of the
+        # streams after every entry (eager steps of models that carry 32-bit streams)
+        self.layer_probe = None
 
     @property
     def graph_safe(self) -> bool:
@@ -71,7 +81,8 @@ class DecoderModel:
             raise ValueError(f"layouts={layouts!r}: use 'auto', 'both' or 'tiled'")
         if layouts == "auto":
             size = torch.finfo(dtype).bits // 8
-            linear = sum(size * math.prod(shape) for name, (shape, role) in full.items() if role == "linear" and name != spec.head_name)
+            linear = sum(size * math.prod(d for d in shape if d is not None) for name, (shape, role) in full.items()
+                         if role == "linear" and name != spec.head_name)
             free = torch.cuda.mem_get_info(self.device)[0]
             layouts = "both" if 2.2 * linear + size * 2 * spec.vocab_size * spec.hidden < 0.8 * free else "tiled"
             if layouts == "tiled" and dtype == torch.bfloat16:
@@ -90,6 +101,8 @@ class DecoderModel:
             else:
                 layer.load(get, dtype, device)
         self.final_norm.load(get, dtype, device)
+        if spec.streams:
+            self._ones = torch.ones(spec.streams, dtype=torch.float32, device=device)
         # whoever runs the model works on a stream of their own: everything that loading enqueued (copies, re-laying of
         # matrices, random draws) is finished before anyone can read it
         torch.cuda.synchronize(self.device)
@@ -118,6 +131,17 @@ class DecoderModel:
         before the last sum.  ``caches[i]`` is the cache view of run-order entry i (its own or the one
         it reads)."""
         n = ctx.n_tokens
+        if self.spec.streams:
+            # copies of the stream in 32-bit, all equal to the embedding's output; blocks update them in place
+            resid = ctx.arena.take((n, self.spec.streams, self.spec.hidden), torch.float32)
+            ops.embed_streams(self.embed, ctx.token_ids, resid, scale=self.spec.embed_scale)
+            for i, call in enumerate(self.spec.run_order):
+                self.layers[call.layer].forward(ctx, resid, None, caches[i], call.cache_from is None, None)
+                if self.layer_probe is not None:
+                    total = torch.empty((n, self.spec.hidden), dtype=torch.float32, device=resid.device)
+                    self.final_norm.read_streams(ctx, resid, self._ones, out=ctx.arena.take((n, self.spec.hidden), self.dtype), sum_out=total)
+                    self.layer_probe(i, total)
+            return resid, None
         resid = ctx.arena.take((n, self.spec.hidden), self.dtype)
         delta = ctx.arena.take((n, self.spec.hidden), self.dtype)
         ops.embed(self.embed, ctx.token_ids, out=resid, scale=self.spec.embed_scale)
@@ -146,7 +170,10 @@ class DecoderModel:
         """32-bit logits [len(rows), vocab] at the given token rows: last sum, last norm and head only there
         (reference: model/llama.py:284-286, engine/engine.py:382)."""
         n = rows.numel()
-        h = self.final_norm.forward(ctx, resid=resid, x=delta, rows=rows, out=ctx.arena.take((n, self.spec.hidden), self.dtype))
+        if self.spec.streams:  # the streams are added up as the last norm reads them
+            h = self.final_norm.read_streams(ctx, resid, self._ones, rows=rows, out=ctx.arena.take((n, self.spec.hidden), self.dtype))
+        else:
+            h = self.final_norm.forward(ctx, resid=resid, x=delta, rows=rows, out=ctx.arena.take((n, self.spec.hidden), self.dtype))
         out = self.head(h, out=ctx.arena.take((n, self.spec.vocab_size), torch.float32), out_f32=True, arena=ctx.arena)
         if self.spec.logit_scale != 1.0 or self.spec.logit_softcap:
             ops.logit_transform(out, self.spec.logit_scale, self.spec.logit_softcap)

@@ -14,10 +14,16 @@ class PagedNeed:
     kv_heads: int
     head_dim: int
     window: int = 0  # 0 = every earlier token stays
+    value_dim: int = 0  # size of a value head if it is not ``head_dim``
+
+    @property
+    def v_dim(self) -> int:
+        return self.value_dim or self.head_dim
 
     @property
     def group_name(self) -> str:
-        return f"kv{self.kv_heads}x{self.head_dim}" + (f"w{self.window}" if self.window else "")
+        return (f"kv{self.kv_heads}x{self.head_dim}" + (f"v{self.value_dim}" if self.value_dim not in (0, self.head_dim) else "")
+                + (f"w{self.window}" if self.window else ""))
 
 
 @dataclass(frozen=True)

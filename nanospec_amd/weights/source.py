@@ -83,10 +83,12 @@ class SafetensorsSource:
 
 def check(source, wanted: dict[str, tuple[int, ...]], optional: set[str] = frozenset()) -> None:
     """Compare a source's header with the tensors a model wants; raise one WeightError that lists
-    everything wrong.  ``optional`` names may be absent (a tied output head)."""
+    everything wrong.  ``optional`` names may be absent (a tied output head).  A wanted size of None fits any size (a part
+    that reads an inner size from the checkpoint itself)."""
     have = set(source.names())
     missing = sorted(n for n in wanted if n not in have and n not in optional)
     unexpected = sorted(have - set(wanted))
-    wrong = [(n, source.shape(n), wanted[n]) for n in sorted(have & set(wanted)) if tuple(source.shape(n)) != tuple(wanted[n])]
+    fits = lambda have_shape, want: len(have_shape) == len(want) and all(w is None or w == h for h, w in zip(have_shape, want))
+    wrong = [(n, source.shape(n), wanted[n]) for n in sorted(have & set(wanted)) if not fits(tuple(source.shape(n)), tuple(wanted[n]))]
     if missing or unexpected or wrong:
         raise WeightError(source.where, missing, unexpected, wrong)
