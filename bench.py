@@ -199,6 +199,79 @@ def serve_ideal_seconds(cfg, esize: int, lens, new_tokens: int, steps: int, dtyp
     return nbytes / (HBM_GBPS * 1e9) + flops / PEAK_FLOPS[dtype]
 
 
+# Sizes for ``--design vuzelix``: the Vuzelix design at the widths, depths and head sizes of the Llama shapes above, beside
+# the Llama model of the same shape.  A quarter of the layers are channel-wise delta-rule layers (16 heads of 128 key and 128
+# value channels, four taps), the others attention layers of the shape's heads with chunks of 1,024 positions and capped
+# scores, every fourth of them on the keys and values of the attention layer before it; dense GELU feed-forwards of the
+# shape's inner size; four hyper-connected streams.
+def vuzelix_config(shape: dict, layers: int | None = None):
+    from dataclasses import replace
+
+    from nanospec_amd.config import VuzelixConfig
+
+    n = layers or shape["num_hidden_layers"]
+    heads, kvh, hd, ff = shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"], shape["intermediate_size"]
+    entries, last_attn = [], None
+    for i in range(n):
+        mlp = {"kind": "dense", "ff": ff}
+        if i % 4 == 0:
+            entries.append({"type": "channel_delta", "mixer": dict(heads=16, kv_heads=16, dim=128, vdim=128, conv=4), "mlp": mlp})
+            continue
+        m = dict(heads=heads, kv_heads=kvh, dim=hd, vdim=hd, scale=hd ** -0.5, softcap=50.0, mask={"size": 1024})
+        if i % 4 == 3 and last_attn is not None:
+            m["kv_from"] = last_attn
+        else:
+            last_attn = i
+        entries.append({"type": "attention", "mixer": m, "mlp": mlp})
+    cfg = VuzelixConfig.from_hf({"architecture": "Vuzelix", "vocab": shape["vocab_size"], "width": shape["hidden_size"],
+                                 "embedding": {"scale": 1.0}, "layers": entries, "norm": {"eps": 1e-5}, "residual_mult": 0.5, "streams": 4,
+                                 "logit_softcap": 30.0})
+    return replace(cfg, decay_rank=64, gate_rank=64)
+
+
+def design_compare(a) -> int:
+    """``--design vuzelix``: prefill and decode throughput of the Vuzelix design beside the Llama model of the same shape,
+    one JSON line.  The default workload and its contract are not touched by this option."""
+    import types
+
+    import torch
+
+    from nanospec_amd import LlamaConfig
+    from nanospec_amd.loader import random_model
+
+    shape = dict(SHAPES[a.shape])
+    if a.layers:
+        shape["num_hidden_layers"] = a.layers
+    dtype = torch.bfloat16 if a.dtype == "bf16" else torch.float32
+    llama = LlamaConfig.from_hf(dict(model_type="llama", **{k: v for k, v in shape.items() if k != "rope_scaling"},
+                                     rope_scaling=dict(rope_type="llama3", **shape["rope_scaling"])))
+    vz = vuzelix_config(shape)
+    out = {}
+    k = min(a.steps, 128)
+    for name, cfg in (("llama", llama), ("vuzelix", vz)):
+        model = random_model(cfg, seed=0, dtype=dtype, on_device=True)
+        facts = types.SimpleNamespace(vocab_size=shape["vocab_size"])
+        row = {}
+        for n in (512, a.prefill_tokens):
+            dt = prefill_run(model, facts, n, 16)
+            row[f"prefill_{n}_tok_s"] = round(n / dt, 1)
+        for b in (1, a.batch):
+            d, c0, c1 = decode_run(model, facts, b, 2048, a.ctx, k, a.warmup, 16, seed=3 + b)
+            row[f"decode_b{b}_ctx{a.ctx}_tok_s"] = round(b * k / d, 1)
+            row[f"decode_b{b}_ms_per_step"] = round(1000 * d / k, 4)
+        out[name] = row
+        del model
+        torch.cuda.empty_cache()
+    ratio = {key: round(out["vuzelix"][key] / out["llama"][key], 3) for key in out["llama"] if key.endswith("tok_s")}
+    print(json.dumps({"metric": f"prefill and decode tok/s of the Vuzelix design beside Llama at the {SHAPE_NAMES[a.shape]} ({a.dtype})",
+                      "unit": "tok/s", "n_gpus": 1, "dtype": a.dtype, "data": "synthetic: random weights, uniform random token ids",
+                      "config": {"shape": SHAPE_NAMES[a.shape], "layers": shape["num_hidden_layers"], "hidden": shape["hidden_size"],
+                                 "vuzelix_layers": [l.type + ("*" if l.kv_from is not None else "") for l in vz.layers], "streams": vz.streams,
+                                 "page_size": 16, "decode_steps": k},
+                      "llama": out["llama"], "vuzelix": out["vuzelix"], "vuzelix_over_llama": ratio}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -215,10 +288,14 @@ def main() -> int:
                     help="instead of the benchmark: continuous batching of this many requests (prompts of 16 to 1,024 tokens, 128 new "
                          "tokens each, prompts in portions of 512)")
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="the benchmark's shape is 8b; the others are for profiles")
+    ap.add_argument("--design", default=None, choices=["vuzelix"],
+                    help="instead of the benchmark: prefill and decode of this design beside the Llama model of the same --shape")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py measures one GPU; this engine has no multi-GPU path (--gpus must be 1)")
         return 2
+    if a.design:
+        return design_compare(a)
 
     import torch
 

@@ -65,7 +65,19 @@ struct AttnParams {
   int near;          // every byte of the key pool and of the value pool lies within 4 GiB of its start, a page's id and a
                      // page's bytes are below 2^24: byte offsets are then 32-bit and one 24-bit multiply-add each
   float scale_log2;  // softmax scale * log2(e)
+  // Options, read only by the kernels instantiated with OPT (every other kernel is compiled as if they did not exist):
+  int chunk;         // > 0: a query sees no key before the start of its own chunk of this many positions
+  int sink;          // the soft-max's denominator holds one more term of score 0
+  float cap;         // > 0: a score s (after the scale) becomes cap * tanh(s / cap); scale_log2 is then log2(e) alone
+  float cap_pre;     // softmax scale / cap
 };
+
+// cap * tanh(x) by one hardware exponential and one reciprocal: tanh(x) = 1 - 2 / (1 + e^(2x)); an exponential that
+// overflows or vanishes gives the limits 1 and -1.
+__device__ __forceinline__ float capped(float raw, float pre, float cap) {
+  const float e = __builtin_amdgcn_exp2f(raw * pre * 2.8853900817779268f);  // e^(2x) = 2^(2x log2 e)
+  return cap - 2.f * cap * __builtin_amdgcn_rcpf(1.f + e);
+}
 
 // 2^x by the hardware instruction alone: arguments here are <= 0, and results below the normal range may flush to 0.
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -103,7 +115,8 @@ struct KVBlock {
 // together fit the memory-side cache they are still there at the next step and plain loads find them, otherwise they only
 // push other data out and non-temporal loads are the faster ones (6.1 against 5.7 TB/s at batch 64 and 3,072 keys of the
 // 8B shape).  The kernel chooses by the number of keys over all layers, which the host leaves in the tiles.
-template <int QT, bool PREFETCH, bool COOP, bool NT>
+// OPT: the options of AttnParams (chunks, capped scores, a sink) are honoured.
+template <int QT, bool PREFETCH, bool COOP, bool NT, bool OPT = false>
 __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
   // what is the same in all lanes of a wave is said to be so (readfirstlane): branches on it are then scalar ones
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -137,6 +150,9 @@ __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
     col_ok[u] = ti < n && hin < G;
     pos[u] = col_ok[u] ? kv_len - n + ti : -1;
     lo[u] = (col_ok[u] && a.window > 0) ? max(0, pos[u] - a.window + 1) : 0;
+    if constexpr (OPT) {
+      if (col_ok[u] && a.chunk > 0) lo[u] = max(lo[u], pos[u] / a.chunk * a.chunk);
+    }
     whi = max(whi, wave_max_i(pos[u]) + 1);                       // keys [wlo, whi) are seen by some column
     wlo = min(wlo, wave_min_i(col_ok[u] ? lo[u] : 0x7fffffff));
     full_hi = min(full_hi, wave_min_i(col_ok[u] ? pos[u] : 0x7fffffff));  // keys <= full_hi are seen by every column
@@ -268,6 +284,12 @@ __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
         } else {
 #pragma unroll
           for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(blk.kn[t * NQ + i], qn[u][i], acc, 0, 0, 0);
+        }
+        if constexpr (OPT) {
+          if (a.cap > 0.f) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] = capped(acc[j], a.cap_pre, a.cap);
+          }
         }
         s[u][t] = acc;
       }
@@ -413,6 +435,9 @@ __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
     // o[u][dt][j] is channel 16 dt + 4 g + j of column c
     if (a.splits == 1) {
       const size_t col = (size_t)(q0 + t0 + tt) * a.heads + head;
+      if constexpr (OPT) {
+        if (a.sink) lsum[u] += fast_exp2(-m[u] * a.scale_log2);  // the term of score 0, in the units of the column's maximum
+      }
       const float inv = 1.f / lsum[u];
 #pragma unroll
       for (int dt = 0; dt < DT; ++dt) {
@@ -434,15 +459,15 @@ __device__ __forceinline__ void attn_tiles(const AttnParams& a) {
 
 constexpr long NT_FROM_BYTES = 192L << 20;  // keys and values of a step (all layers) from which non-temporal loads pay
 
-template <int QT, bool PREFETCH, bool COOP>
+template <int QT, bool PREFETCH, bool COOP, bool OPT = false>
 __global__ __launch_bounds__(256) void attn_mfma_kernel(AttnParams a) {
   if constexpr (QT == 1) {
     // decode tiles carry the number of keys that the step's decode rows read over all layers (the same in every tile)
     const long bytes = (long)a.tiles[5] * a.kv_heads * HD * 4;
-    if (bytes >= NT_FROM_BYTES) attn_tiles<QT, PREFETCH, COOP, true>(a);
-    else attn_tiles<QT, PREFETCH, COOP, false>(a);
+    if (bytes >= NT_FROM_BYTES) attn_tiles<QT, PREFETCH, COOP, true, OPT>(a);
+    else attn_tiles<QT, PREFETCH, COOP, false, OPT>(a);
   } else {
-    attn_tiles<QT, PREFETCH, COOP, false>(a);
+    attn_tiles<QT, PREFETCH, COOP, false, OPT>(a);
   }
 }
 
@@ -971,7 +996,7 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
 // results are addressed by tile, so nothing here waits for the tile descriptor except the final store.
 __global__ __launch_bounds__(64) void attn_reduce_kernel(bf16_t* __restrict__ out, const float* __restrict__ part_o,
                                                          const float* __restrict__ part_ml, const int* __restrict__ tiles,
-                                                         int heads, int tile_tokens, int splits) {
+                                                         int heads, int tile_tokens, int splits, int sink) {
   const int tile = blockIdx.x, head = blockIdx.y, tt = blockIdx.z;
   const int lane = threadIdx.x;
   const size_t pcol = ((size_t)tile * tile_tokens + tt) * heads + head;
@@ -993,6 +1018,7 @@ __global__ __launch_bounds__(64) void attn_reduce_kernel(bf16_t* __restrict__ ou
   float l = ls * wgt;
 #pragma unroll
   for (int o = 32; o > 0; o >>= 1) l += __shfl_xor(l, o, 64);
+  if (sink) l += exp2f(-mstar);  // the term of score 0 (the ranges' maxima are in the exponent's units)
   const float inv = 1.f / l;
   float acc[PER];
 #pragma unroll
@@ -1048,7 +1074,8 @@ extern "C" int ns_attn_prompt_form(void) { return prompt_form(); }
 extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* q, int q_stride, const void* k_cache,
                             const void* v_cache, const int* tiles, const int* block_table, int table_stride, int n_tiles,
                             int heads, int kv_heads, int page_size, int hp, int splits, int window, float scale, int qt,
-                            int coop, long pool_pages, hipStream_t stream) {
+                            int coop, long pool_pages, int chunk, float cap, int sink, hipStream_t stream) {
+  if (chunk < 0 || cap < 0.f) return NS_ERR_BAD_ARG;
   if (n_tiles <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || page_size != PS || window < 0 ||
       splits < 1 || splits > 64 || (q_stride & 7) || ((uintptr_t)tiles & 15))
     return NS_ERR_BAD_ARG;
@@ -1066,11 +1093,22 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   const long page_bytes = (long)kv_heads * HD * PS * 2;
   a.near = pool_pages > 0 && pool_pages < (1L << 24) && page_bytes < (1L << 24) && pool_pages * page_bytes <= (1L << 32);
   a.scale_log2 = scale * 1.4426950408889634f;
+  // chunks, capped scores and a sink are honoured by the kernels that walk tiles without sharing keys through LDS
+  const bool opt = chunk > 0 || cap > 0.f || sink != 0;
+  a.chunk = chunk; a.sink = sink; a.cap = cap; a.cap_pre = cap > 0.f ? scale / cap : 0.f;
+  if (cap > 0.f) a.scale_log2 = 1.4426950408889634f;  // the scale is applied where the scores are capped
   const int G = heads / kv_heads;
   const long items = (long)n_tiles * splits * kv_heads * ((G + hp - 1) / hp);
   const long blocks = coop ? items : (items + 3) / 4;
   if (blocks > 0x7fffffffL) return NS_ERR_BAD_ARG;
-  if (qt == 2 && SHARED_OK) {
+  if (opt) {
+    if (qt == 2)
+      attn_mfma_kernel<2, false, false, true><<<(unsigned)blocks, 256, 0, stream>>>(a);
+    else if (coop)
+      attn_mfma_kernel<1, true, true, true><<<(unsigned)blocks, 256, 0, stream>>>(a);
+    else
+      attn_mfma_kernel<1, true, false, true><<<(unsigned)blocks, 256, 0, stream>>>(a);
+  } else if (qt == 2 && SHARED_OK) {
     const long wgs = (long)n_tiles * splits * kv_heads * ((G + 3) / 4);
     if (wgs > 0x7fffffffL) return NS_ERR_BAD_ARG;
 #ifndef NS_PREFILL16
@@ -1096,6 +1134,6 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   if (heads > 65535) return NS_ERR_BAD_ARG;
   const int tile_tokens = qt * 16 / hp;
   attn_reduce_kernel<<<dim3(n_tiles, heads, tile_tokens), 64, 0, stream>>>((bf16_t*)out, (const float*)part_o, (const float*)part_ml,
-                                                                           tiles, heads, tile_tokens, splits);
+                                                                           tiles, heads, tile_tokens, splits, sink);
   return ns_launch_status();
 }

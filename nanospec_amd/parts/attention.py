@@ -87,11 +87,12 @@ class LaunchPlan:
     coop: bool = False
 
 
-def launch_plans(ctx, group: int, kv_heads: int, head_dim: int) -> list[LaunchPlan]:
+def launch_plans(ctx, group: int, kv_heads: int, head_dim: int, span: int = 0) -> list[LaunchPlan]:
     """How the matrix-core attention kernel is launched for a mixer with ``group`` query heads per key/value head, over
     the tile lists of the batch: prompt portions as 32-token tiles of one head, their keys cut into ranges when there
     are too few tiles to fill the GPU and many keys (a short portion late in a long prompt); decode rows with all heads
-    of a group in one tile and the keys cut into ranges so that the launch fills the GPU."""
+    of a group in one tile and the keys cut into ranges so that the launch fills the GPU.  ``span`` > 0: no query sees more
+    than this many keys (a chunked mask), whatever the rows' lengths."""
     plans = []  # made afresh per call: the workspace lives in the caller's arena scope
     units = ops.compute_units(ctx.token_ids.device)
     chunk_tiles, decode_tiles = TilePlan.views(ctx)
@@ -99,7 +100,7 @@ def launch_plans(ctx, group: int, kv_heads: int, head_dim: int) -> list[LaunchPl
     if n_chunk_tiles:
         tokens = TilePlan.TOKENS
         wgs = n_chunk_tiles * kv_heads * -(-group // 4)
-        blocks = -(-ctx.max_chunk_kv // 32)
+        blocks = -(-(min(ctx.max_chunk_kv, span + tokens) if span else ctx.max_chunk_kv) // 32)
         # fewer workgroups than compute units (one fits a unit): cut the keys into ranges
         splits = max(1, min(16, units // wgs, blocks // PORTION_RANGE_BLOCKS))
         ws = None
@@ -120,10 +121,11 @@ def launch_plans(ctx, group: int, kv_heads: int, head_dim: int) -> list[LaunchPl
         # keys 86 against 132 us a layer; the kernel leaves the ranges beyond the sixteenth empty for shorter rows,
         # and where no request can be that long they are not launched: they would cost a captured step 1%)
         items = n_decode_tiles * kv_heads * -(-group // hp)
-        splits = max(1, min(32 if ctx.max_kv_len >= LONG_ROW_KEYS else 16, DECODE_WAVES_PER_UNIT * units // (4 * items)))
+        longest = min(ctx.max_kv_len, span) if span else ctx.max_kv_len
+        splits = max(1, min(32 if longest >= LONG_ROW_KEYS else 16, DECODE_WAVES_PER_UNIT * units // (4 * items)))
         # never ranges of fewer than 256 keys (in a captured step: of what its block tables can hold): short rows are
         # short chains already, and a single range needs no kernel to join it
-        splits = max(1, min(splits, -(-ctx.max_kv_len // 256)))
+        splits = max(1, min(splits, -(-longest // 256)))
         ws = None
         if splits > 1:
             cols = n_decode_tiles * (16 // hp) * kv_heads * group
@@ -274,8 +276,15 @@ class Attention:
             ops.unit_kv_write(qkv, ctx.positions, ctx.token_req, table, cache.k, cache.v, s.heads, s.kv_heads, s.head_dim, s.v_dim,
                               s.qk_norm_eps, own_kv=s.own_kv)
         att = ctx.arena.take((n, s.heads * s.v_dim), x.dtype)
-        ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads, s.head_dim,
-                              s.softmax_scale, window=s.window, v_dim=s.v_dim, chunk=s.chunk, cap=s.score_cap, sink=s.sink)
+        if s.v_dim == s.head_dim and ops.mfma_attention_takes(x.dtype, s.head_dim, cache.k.shape[2]):
+            # bfloat16 on the matrix cores: the tile kernels honour chunks, capped scores and the sink
+            for plan in launch_plans(ctx, s.heads // s.kv_heads, s.kv_heads, s.head_dim, span=s.chunk):
+                ops.attention_mfma(qkv, att, cache.k, cache.v, plan.tiles, table, s.heads, s.kv_heads, s.head_dim, s.softmax_scale,
+                                   window=s.window, hp=plan.hp, splits=plan.splits, workspace=plan.workspace, qt=plan.qt, coop=plan.coop,
+                                   chunk=s.chunk, cap=s.score_cap, sink=s.sink)
+        else:
+            ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads, s.head_dim,
+                                  s.softmax_scale, window=s.window, v_dim=s.v_dim, chunk=s.chunk, cap=s.score_cap, sink=s.sink)
         if residual is not None:
             return self.wo.into_residual(att, residual, arena=ctx.arena, plain_copy=not ctx.captured)
         return self.wo(att, out=out, arena=ctx.arena, plain_copy=not ctx.captured)

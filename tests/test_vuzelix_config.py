@@ -1,0 +1,167 @@
+"""The Vuzelix configuration as data (no GPU): what config.json's keys become, what is refused, and a few properties that
+pin the plain implementation the GPU tests compare with."""
+
+from __future__ import annotations
+
+import math
+from dataclasses import replace
+
+import pytest
+import torch
+
+import plain_vuzelix as pv
+
+CFG = {"architecture": "Vuzelix", "vocab": 90, "width": 48, "embedding": {"scale": 1.5}, "norm": {"eps": 1e-5}, "residual_mult": 0.25,
+       "streams": 2, "logit_softcap": 12.0,
+       "layers": [{"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 8, "vdim": 12, "scale": 0.5, "softcap": 9.0,
+                                                   "mask": {"size": 10}}, "mlp": {"kind": "dense", "ff": 64}},
+                  {"type": "channel_delta", "mixer": {"heads": 2, "kv_heads": 1, "dim": 8, "vdim": 12, "conv": 3}, "mlp": None},
+                  {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 8, "vdim": 12, "scale": 0.25, "kv_from": 0},
+                   "mlp": {"kind": "dense", "ff": 32}}]}
+
+
+def test_keys_become_specs():
+    from nanospec_amd.config import resolve
+    from nanospec_amd.config.spec import AttentionSpec, ChannelDeltaSpec, DenseFFSpec, StreamBlockSpec
+
+    config, spec = resolve(CFG)
+    assert (spec.vocab_size, spec.hidden, spec.streams, spec.embed_scale, spec.logit_softcap) == (90, 48, 2, 1.5, 12.0)
+    assert (spec.embed_name, spec.head_name, spec.final_norm_name) == ("embed", "head", "final.norm")
+    assert [(c.layer, c.cache_from) for c in spec.run_order] == [(0, None), (1, None), (2, 0)]
+    a, d, b = spec.layers
+    assert all(isinstance(x, StreamBlockSpec) and x.streams == 2 and x.mult == 0.25 for x in spec.layers)
+    assert isinstance(a.mixer, AttentionSpec) and (a.mixer.head_dim, a.mixer.v_dim, a.mixer.chunk, a.mixer.score_cap) == (8, 12, 10, 9.0)
+    assert a.mixer.sink and a.mixer.own_kv and a.mixer.qk_norm_eps == 1e-5 and a.mixer.softmax_scale == 0.5 and a.mixer.general
+    assert (b.mixer.own_kv, b.mixer.chunk, b.mixer.score_cap, b.mixer.softmax_scale) == (False, 0, 0.0, 0.25)
+    assert isinstance(d.mixer, ChannelDeltaSpec) and (d.mixer.key_dim, d.mixer.value_dim, d.mixer.conv) == (8, 12, 3)
+    assert d.ffn is None and d.ffn_norm is None and isinstance(a.ffn, DenseFFSpec) and a.ffn.intermediate == 64
+    assert config.to_hf()["layers"] == CFG["layers"] and type(config).from_hf(config.to_hf()) == config
+
+
+def test_absent_keys_do_nothing():
+    from nanospec_amd.config import resolve
+
+    cfg = {k: v for k, v in CFG.items() if k not in ("embedding", "residual_mult", "streams", "logit_softcap")}
+    _, spec = resolve(cfg)
+    assert (spec.streams, spec.embed_scale, spec.logit_softcap) == (1, 1.0, 0.0)
+    assert all(b.streams == 0 and b.mult == 1.0 for b in spec.layers)
+
+
+def test_tensor_names_and_shapes():
+    from nanospec_amd.config import VuzelixConfig
+    from nanospec_amd.parts import wanted_tensors
+
+    spec = replace(VuzelixConfig.from_hf(CFG), decay_rank=6, gate_rank=5).model_spec()
+    shapes = {k: v[0] for k, v in wanted_tensors(spec).items()}
+    assert shapes["l0.mix.q"] == (32, 48) and shapes["l0.mix.k"] == (16, 48) and shapes["l0.mix.v"] == (24, 48) and shapes["l0.mix.o"] == (48, 48)
+    assert "l2.mix.k" not in shapes and "l2.mix.v" not in shapes and shapes["l2.mix.q"] == (32, 48)
+    assert shapes["l1.mix.q.conv"] == (8, 3) and shapes["l1.mix.v.conv"] == (24, 3) and shapes["l1.mix.a1"] == (6, 48)
+    assert shapes["l1.mix.a2"] == (16, 6) and shapes["l1.mix.g2"] == (24, 5) and shapes["l1.mix.A_log"] == (2,) and shapes["l1.mix.norm"] == (12,)
+    assert shapes["l0.hc1.mix"] == (2, 2) and shapes["l0.hc2.in"] == (2,) and "l1.hc2.in" not in shapes and "l1.norm2" not in shapes
+    # without ranks the inner sizes are left to the checkpoint
+    open_shapes = {k: v[0] for k, v in wanted_tensors(VuzelixConfig.from_hf(CFG).model_spec()).items()}
+    assert open_shapes["l1.mix.a1"] == (None, 48) and open_shapes["l1.mix.g2"] == (24, None)
+
+
+@pytest.mark.parametrize("change,match", [
+    (lambda c: c["layers"][0].update(type="conv"), "unknown mixer"),
+    (lambda c: c["layers"][2]["mixer"].update(kv_from=1), "keys and values"),
+    (lambda c: c["layers"][2]["mixer"].update(kv_from=2), "keys and values"),
+    (lambda c: c["layers"][2]["mixer"].update(dim=16), "differ"),
+    (lambda c: c["layers"][0]["mixer"].update(heads=3), "heads"),
+    (lambda c: c.update(streams=0), "streams"),
+    (lambda c: c["layers"][0]["mlp"].update(kind="routed"), "feed-forward"),
+])
+def test_refusals(change, match):
+    import copy
+
+    from nanospec_amd.config import resolve
+
+    cfg = copy.deepcopy(CFG)
+    change(cfg)
+    with pytest.raises(ValueError, match=match):
+        resolve(cfg)
+
+
+def test_weights_with_an_inner_size_of_their_own_fit():
+    from nanospec_amd.weights import WeightError, check
+
+    class Header:
+        where = "<header>"
+
+        def __init__(self, shapes):
+            self.shapes = shapes
+
+        def names(self):
+            return list(self.shapes)
+
+        def shape(self, name):
+            return self.shapes[name]
+
+    check(Header({"a": (7, 48)}), {"a": (None, 48)})
+    with pytest.raises(WeightError):
+        check(Header({"a": (7, 40)}), {"a": (None, 48)})
+
+
+# ------------------------------------------------------------------------------------------------ the plain implementation
+
+
+def test_plain_delta_rule_is_a_lossless_memory_without_decay():
+    T, D, E = 6, 8, 3
+    k = torch.eye(D, dtype=torch.float64)[:T].view(T, 1, D)
+    v = torch.randn(T, 1, E, dtype=torch.float64)
+    q = k.flip(0)  # token t asks for what token T-1-t wrote: known only in the second half
+    o, S = pv.delta_recurrence(q, k, v, torch.ones(T, 1, dtype=torch.float64), torch.ones(T, 1, D, dtype=torch.float64))
+    assert o[: T // 2].abs().max() == 0 and torch.allclose(o[T // 2 :], v.flip(0)[T // 2 :])
+    # a write strength of 0 writes nothing; a decay of 0 forgets everything but the current token
+    o0, _ = pv.delta_recurrence(q, k, v, torch.zeros(T, 1, dtype=torch.float64), torch.ones(T, 1, D, dtype=torch.float64))
+    assert o0.abs().max() == 0
+    o1, _ = pv.delta_recurrence(k, k, v, torch.ones(T, 1, dtype=torch.float64), torch.zeros(T, 1, D, dtype=torch.float64))
+    assert torch.allclose(o1, v)
+
+
+def test_plain_convolution_is_causal_and_ends_in_the_current_token():
+    x = torch.randn(9, 4, dtype=torch.float64)
+    taps = torch.randn(4, 3, dtype=torch.float64)
+    y = pv.causal_conv_silu(x, taps)
+    z = x[0] * taps[:, 2]
+    assert torch.allclose(y[0], z * torch.sigmoid(z))
+    x2 = x.clone()
+    x2[5:] += 1.0
+    assert torch.equal(pv.causal_conv_silu(x2, taps)[:5], y[:5])
+
+
+def test_plain_attention_mask_and_sink():
+    torch.manual_seed(0)
+    m = {"heads": 2, "kv_heads": 1, "dim": 4, "vdim": 3, "scale": 0.5, "mask": {"size": 4}}
+    w = {"q": torch.randn(8, 6, dtype=torch.float64), "o": torch.eye(6, dtype=torch.float64)}
+    h = torch.randn(10, 6, dtype=torch.float64)
+    k, v = torch.randn(10, 1, 4, dtype=torch.float64), torch.randn(10, 1, 3, dtype=torch.float64)
+    out = pv.attention(h, w, "", m, 1e-5, (k, v))
+    v2 = v.clone()
+    v2[:4] += 5.0  # keys of the first chunk are nothing to the later ones
+    assert torch.equal(pv.attention(h, w, "", m, 1e-5, (k, v2))[4:], out[4:])
+    # position 4 sees only itself: its value times e^s / (1 + e^s)
+    q = pv.rms((h @ w["q"].T).view(10, 2, 4), 1e-5)
+    s = (q[4] * k[4]).sum(-1) * 0.5
+    assert torch.allclose(out[4].view(2, 3), (torch.exp(s) / (1 + torch.exp(s))).view(2, 1) * v[4])
+
+
+def test_plain_model_without_streams_is_a_plain_residual():
+    """With one hyper-connected stream whose tensors are all 1 the model equals the one without the key."""
+    torch.manual_seed(1)
+    cfg = {k: v for k, v in CFG.items() if k != "streams"}
+    from nanospec_amd.config import VuzelixConfig
+    from nanospec_amd.parts import wanted_tensors
+    from nanospec_amd.weights import random_tensors
+
+    conf = replace(VuzelixConfig.from_hf(cfg), decay_rank=4, gate_rank=4)
+    w = random_tensors(wanted_tensors(conf.model_spec()), 0)
+    toks = [3, 1, 4, 1, 5, 9, 2, 6, 5, 3, 5, 8, 9, 7]
+    base = pv.forward(cfg, w, toks)
+    one = dict(w)
+    for l, layer in enumerate(cfg["layers"]):
+        for q in (1, 2) if layer["mlp"] else (1,):
+            one[f"l{l}.hc{q}.in"], one[f"l{l}.hc{q}.out"], one[f"l{l}.hc{q}.mix"] = torch.ones(1), torch.ones(1), torch.ones(1, 1)
+    assert torch.allclose(pv.forward({**cfg, "streams": 1}, one, toks), base)
+    assert base.abs().max() < 12.0 and not math.isnan(float(base.sum()))
