@@ -124,106 +124,155 @@ extern "C" int ns_delta_prep(float* qkv, int C, float* g, float* beta, const voi
 // ------------------------------------------------------------------------------------------------
 // The recurrence.  grid (requests, heads, blocks of columns); a thread = (column jl of the block, row group rg), lane
 // = jl * RG + rg, RG a power of two (at most 64) with 16 RG >= D.  Channels beyond D carry zeros.
+//
+// A token's step is a chain (decay, dot product, lane exchange, update, dot product, lane exchange) that cannot start
+// before the token's operands are there, so the operands of the next ND_STAGE_FLOATS floats' worth of tokens are
+// fetched by the whole workgroup at once (coalesced, all loads in flight together), parked in registers while the
+// current stage's tokens are worked through from LDS, and then written to the other LDS buffer.  The arithmetic of a
+// token is the same whatever the stage it falls into: results do not depend on how a prompt was cut.
 // ------------------------------------------------------------------------------------------------
-struct DeltaVec {
-  float v[ND_ROWS];
-};
-
-__device__ __forceinline__ void delta_load(DeltaVec& out, const float* p, int valid, bool vec4) {
-  if (vec4 && valid == ND_ROWS) {
-    const float4* p4 = reinterpret_cast<const float4*>(p);
-#pragma unroll
-    for (int i = 0; i < ND_ROWS / 4; ++i) {
-      const float4 t = p4[i];
-      out.v[4 * i] = t.x, out.v[4 * i + 1] = t.y, out.v[4 * i + 2] = t.z, out.v[4 * i + 3] = t.w;
-    }
-  } else {
-#pragma unroll
-    for (int i = 0; i < ND_ROWS; ++i) out.v[i] = i < valid ? p[i] : 0.f;
-  }
-}
-
 __device__ __forceinline__ float group_sum(float v, int rg_count) {
   for (int o = 1; o < rg_count; o <<= 1) v += __shfl_xor(v, o, NS_WAVE);
   return v;
 }
 
-__global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, const float* __restrict__ qkv, int C,
+#define ND_STAGE_FLOATS 6144                       // floats of one stage in LDS (two stages are held)
+#define ND_STAGE_REGS (ND_STAGE_FLOATS / 256)      // of which each of the 256 threads fetches this many
+
+struct DeltaShape {
+  int C, H, G, D, E, RG, Dp, dp_shift, cols, tok_stride, stage_tokens;
+};
+
+__global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, const float* __restrict__ qkv,
                                                          const float* __restrict__ g, const float* __restrict__ beta,
                                                          float* __restrict__ state, size_t slot_stride, const int* __restrict__ qo_indptr,
-                                                         const int* __restrict__ state_slots, int H, int G, int D, int E, int RG, int vec4) {
+                                                         const int* __restrict__ state_slots, DeltaShape p) {
+  __shared__ __attribute__((aligned(16))) float stage[2][ND_STAGE_FLOATS];
   const int b = blockIdx.x, h = blockIdx.y;
   const int r0 = qo_indptr[b], r1 = qo_indptr[b + 1];
   if (r1 <= r0) return;
-  const int cols = blockDim.x / RG;
+  const int D = p.D, E = p.E, RG = p.RG;
   const int jl = threadIdx.x / RG, rg = threadIdx.x % RG;
-  const int j = blockIdx.z * cols + jl;
+  const int j0 = blockIdx.z * p.cols, j = j0 + jl;
   const bool col_ok = j < E;
   const int d0 = rg * ND_ROWS;
-  const int valid = max(0, min(ND_ROWS, D - d0));
-  const int kh = h / (H / G);
+  const int kh = h / (p.H / p.G);
   float* S = state + (size_t)state_slots[b] * slot_stride + (size_t)h * D * E;
   float s[ND_ROWS];
 #pragma unroll
-  for (int i = 0; i < ND_ROWS; ++i) s[i] = (col_ok && i < valid) ? S[(size_t)(d0 + i) * E + j] : 0.f;
-  const size_t q_off = (size_t)kh * D + d0, k_off = (size_t)G * D + (size_t)kh * D + d0, v_off = (size_t)2 * G * D + (size_t)h * E + (col_ok ? j : 0);
-  const size_t g_off = (size_t)h * D + d0;
-  const bool v4 = vec4 != 0;
-  DeltaVec qn, kn, gn;
-  float vn, bn;
-  {
-    const float* row = qkv + (size_t)r0 * C;
-    delta_load(qn, row + q_off, valid, v4);
-    delta_load(kn, row + k_off, valid, v4);
-    delta_load(gn, g + (size_t)r0 * H * D + g_off, valid, v4);
-    vn = row[v_off];
-    bn = beta[(size_t)r0 * H + h];
-  }
-  for (int r = r0; r < r1; ++r) {
-    const DeltaVec qc = qn, kc = kn, gc = gn;
-    const float vc = vn, bc = bn;
-    if (r + 1 < r1) {  // the next token's operands are on their way while this one's chain runs
-      const float* row = qkv + (size_t)(r + 1) * C;
-      delta_load(qn, row + q_off, valid, v4);
-      delta_load(kn, row + k_off, valid, v4);
-      delta_load(gn, g + (size_t)(r + 1) * H * D + g_off, valid, v4);
-      vn = row[v_off];
-      bn = beta[(size_t)(r + 1) * H + h];
-    }
-    float dot = 0.f;
+  for (int i = 0; i < ND_ROWS; ++i) s[i] = (col_ok && d0 + i < D) ? S[(size_t)(d0 + i) * E + j] : 0.f;
+
+  // what element e of a stage that starts at row `first` is: token e / tok_stride, then q [Dp] | k [Dp] | g [Dp] | v [cols] | beta
+  const float* q_src = qkv + (size_t)kh * D;
+  const float* k_src = qkv + (size_t)p.G * D + (size_t)kh * D;
+  const float* v_src = qkv + (size_t)2 * p.G * D + (size_t)h * E + j0;
+  const float* g_src = g + (size_t)h * D;
+  const int stage_elems = p.stage_tokens * p.tok_stride;
+  auto fetch = [&](float (&regs)[ND_STAGE_REGS], int first) {
+    int tt = threadIdx.x / p.tok_stride, off = threadIdx.x - tt * p.tok_stride;  // of element e, kept up as e grows by 256
 #pragma unroll
-    for (int i = 0; i < ND_ROWS; ++i) {
-      s[i] *= gc.v[i];
-      dot = fmaf(kc.v[i], s[i], dot);
+    for (int i = 0; i < ND_STAGE_REGS; ++i) {
+      const int e = threadIdx.x + i * 256;
+      float val = 0.f;
+      if (e < stage_elems) {
+        const int r = first + tt;
+        if (r < r1) {
+          const int part = off >> p.dp_shift, d = off & (p.Dp - 1);
+          if (part < 3) {
+            if (d < D) val = part == 0 ? q_src[(size_t)r * p.C + d] : (part == 1 ? k_src[(size_t)r * p.C + d] : g_src[(size_t)r * p.H * D + d]);
+          } else {
+            const int c = off - 3 * p.Dp;
+            if (c < p.cols) val = j0 + c < E ? v_src[(size_t)r * p.C + c] : 0.f;
+            else if (c == p.cols) val = beta[(size_t)r * p.H + h];
+          }
+        }
+      }
+      regs[i] = val;
+      off += 256;
+      while (off >= p.tok_stride) off -= p.tok_stride, ++tt;
     }
-    dot = group_sum(dot, RG);
-    const float u = bc * (vc - dot);
-    float out = 0.f;
+  };
+  auto park = [&](const float (&regs)[ND_STAGE_REGS], float* buf) {
 #pragma unroll
-    for (int i = 0; i < ND_ROWS; ++i) {
-      s[i] = fmaf(kc.v[i], u, s[i]);
-      out = fmaf(qc.v[i], s[i], out);
+    for (int i = 0; i < ND_STAGE_REGS; ++i) {
+      const int e = threadIdx.x + i * 256;
+      if (e < stage_elems) buf[e] = regs[i];
     }
-    out = group_sum(out, RG);
-    if (rg == 0 && col_ok) o[(size_t)r * H * E + (size_t)h * E + j] = out;
+  };
+
+  float regs[ND_STAGE_REGS];
+  fetch(regs, r0);
+  park(regs, stage[0]);
+  __syncthreads();
+  int cur = 0;
+  for (int first = r0; first < r1; first += p.stage_tokens) {
+    const bool more = first + p.stage_tokens < r1;
+    if (more) fetch(regs, first + p.stage_tokens);
+    const float* buf = stage[cur];
+    const int n = min(p.stage_tokens, r1 - first);
+    for (int tt = 0; tt < n; ++tt) {
+      const float* tok = buf + tt * p.tok_stride;
+      const float4* q4 = reinterpret_cast<const float4*>(tok + d0);
+      const float4* k4 = reinterpret_cast<const float4*>(tok + p.Dp + d0);
+      const float4* g4 = reinterpret_cast<const float4*>(tok + 2 * p.Dp + d0);
+      const float vc = tok[3 * p.Dp + jl], bc = tok[3 * p.Dp + p.cols];
+      float kk[ND_ROWS];
+      float part[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < ND_ROWS / 4; ++i) {
+        const float4 gv = g4[i], kv = k4[i];
+        kk[4 * i] = kv.x, kk[4 * i + 1] = kv.y, kk[4 * i + 2] = kv.z, kk[4 * i + 3] = kv.w;
+        s[4 * i] *= gv.x, s[4 * i + 1] *= gv.y, s[4 * i + 2] *= gv.z, s[4 * i + 3] *= gv.w;
+        part[0] = fmaf(kv.x, s[4 * i], part[0]);
+        part[1] = fmaf(kv.y, s[4 * i + 1], part[1]);
+        part[2] = fmaf(kv.z, s[4 * i + 2], part[2]);
+        part[3] = fmaf(kv.w, s[4 * i + 3], part[3]);
+      }
+      const float dot = group_sum((part[0] + part[1]) + (part[2] + part[3]), RG);
+      const float u = bc * (vc - dot);
+      float acc[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int i = 0; i < ND_ROWS / 4; ++i) {
+        const float4 qv = q4[i];
+        s[4 * i] = fmaf(kk[4 * i], u, s[4 * i]);
+        s[4 * i + 1] = fmaf(kk[4 * i + 1], u, s[4 * i + 1]);
+        s[4 * i + 2] = fmaf(kk[4 * i + 2], u, s[4 * i + 2]);
+        s[4 * i + 3] = fmaf(kk[4 * i + 3], u, s[4 * i + 3]);
+        acc[0] = fmaf(qv.x, s[4 * i], acc[0]);
+        acc[1] = fmaf(qv.y, s[4 * i + 1], acc[1]);
+        acc[2] = fmaf(qv.z, s[4 * i + 2], acc[2]);
+        acc[3] = fmaf(qv.w, s[4 * i + 3], acc[3]);
+      }
+      const float out = group_sum((acc[0] + acc[1]) + (acc[2] + acc[3]), RG);
+      if (rg == 0 && col_ok) o[(size_t)(first + tt) * p.H * E + (size_t)h * E + j] = out;
+    }
+    if (more) park(regs, stage[cur ^ 1]);
+    __syncthreads();
+    cur ^= 1;
   }
 #pragma unroll
   for (int i = 0; i < ND_ROWS; ++i)
-    if (col_ok && i < valid) S[(size_t)(d0 + i) * E + j] = s[i];
+    if (col_ok && d0 + i < D) S[(size_t)(d0 + i) * E + j] = s[i];
 }
 
 extern "C" int ns_delta_scan(float* o, const float* qkv, int C, const float* g, const float* beta, float* state, size_t slot_stride,
                              const int* qo_indptr, const int* state_slots, int n_reqs, int H, int G, int D, int E, hipStream_t stream) {
   if (n_reqs <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || D > ND_ROWS * NS_WAVE || E <= 0 || H > 65535) return NS_ERR_BAD_ARG;
-  int RG = 1;
-  while (RG * ND_ROWS < D) RG *= 2;
-  const int cols = 256 / RG;
-  const int zb = (E + cols - 1) / cols;
+  DeltaShape p;
+  p.C = C, p.H = H, p.G = G, p.D = D, p.E = E;
+  p.RG = 1;
+  while (p.RG * ND_ROWS < D) p.RG *= 2;
+  p.Dp = p.RG * ND_ROWS;
+  p.dp_shift = 0;
+  while ((1 << p.dp_shift) < p.Dp) ++p.dp_shift;
+  p.cols = 256 / p.RG;
+  p.tok_stride = 3 * p.Dp + ((p.cols + 1 + 3) / 4) * 4;
+  p.stage_tokens = ND_STAGE_FLOATS / p.tok_stride;
+  if (p.stage_tokens < 1) return NS_ERR_BAD_ARG;
+  if (p.stage_tokens > 64) p.stage_tokens = 64;
+  const int zb = (E + p.cols - 1) / p.cols;
   if (zb > 65535) return NS_ERR_BAD_ARG;
-  // 16-byte loads where every vector a thread reads starts at a multiple of four floats
-  const int vec4 = (D % 4 == 0 && C % 4 == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)g % 16) == 0) ? 1 : 0;
-  delta_scan_kernel<<<dim3(n_reqs, H, zb), 256, 0, stream>>>(o, qkv, C, g, beta, state, slot_stride, qo_indptr, state_slots, H, G, D, E, RG,
-                                                              vec4);
+  delta_scan_kernel<<<dim3(n_reqs, H, zb), 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p);
   return ns_launch_status();
 }
 

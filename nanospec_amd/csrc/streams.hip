@@ -108,6 +108,112 @@ extern "C" int ns_stream_write(float* x, const float* mix, const float* gain, co
   return ns_launch_status();
 }
 
+// The two in one pass with 16-byte accesses, for S <= 4 streams and rows of a multiple of four up to 8,192 columns: the
+// write of one sublayer's output (``y`` given) followed by the read for the next sublayer (``coeff`` given), each
+// optional.  A thread keeps its columns of the mix u in registers between the sum of squares and the output, so a row is
+// read once.  ``store`` = 0 leaves x as it was (the last read of a step, whose written streams nobody reads again).
+template <typename T, int S, int KMAX>
+__global__ __launch_bounds__(256) void stream_step_kernel(float* __restrict__ x, const float* __restrict__ mix, const float* __restrict__ gain,
+                                                          const T* __restrict__ y, int y_stride, const float* __restrict__ coeff,
+                                                          const T* __restrict__ w, const int* __restrict__ rows, T* __restrict__ out,
+                                                          float* __restrict__ sum_out, int W, float eps, int store) {
+  __shared__ float scratch[16];
+  const int i = blockIdx.x;
+  const size_t r = rows ? (size_t)rows[i] : (size_t)i;
+  float* xr = x + r * S * W;
+  float m[S][S], gn[S], a[S];
+#pragma unroll
+  for (int s = 0; s < S; ++s) {
+    gn[s] = y ? gain[s] : 0.f;
+    a[s] = coeff ? coeff[s] : 0.f;
+#pragma unroll
+    for (int t = 0; t < S; ++t) m[s][t] = y ? mix[s * S + t] : (s == t ? 1.f : 0.f);
+  }
+  float4 u[KMAX];
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    const int c = (threadIdx.x + k * 256) * 4;
+    if (c < W) {
+      float4 v[S];
+#pragma unroll
+      for (int s = 0; s < S; ++s) v[s] = *reinterpret_cast<const float4*>(xr + (size_t)s * W + c);
+      if (y) {
+        const T* yp = y + r * y_stride + c;
+        const float4 yv = {to_f(yp[0]), to_f(yp[1]), to_f(yp[2]), to_f(yp[3])};
+        float4 nv[S];
+#pragma unroll
+        for (int t = 0; t < S; ++t) {
+          float4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+          for (int s = 0; s < S; ++s) {
+            acc.x = fmaf(m[s][t], v[s].x, acc.x), acc.y = fmaf(m[s][t], v[s].y, acc.y);
+            acc.z = fmaf(m[s][t], v[s].z, acc.z), acc.w = fmaf(m[s][t], v[s].w, acc.w);
+          }
+          nv[t] = {fmaf(gn[t], yv.x, acc.x), fmaf(gn[t], yv.y, acc.y), fmaf(gn[t], yv.z, acc.z), fmaf(gn[t], yv.w, acc.w)};
+        }
+#pragma unroll
+        for (int t = 0; t < S; ++t) {
+          v[t] = nv[t];
+          if (store) *reinterpret_cast<float4*>(xr + (size_t)t * W + c) = nv[t];
+        }
+      }
+      float4 mixv = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s = 0; s < S; ++s) {
+        mixv.x = fmaf(a[s], v[s].x, mixv.x), mixv.y = fmaf(a[s], v[s].y, mixv.y);
+        mixv.z = fmaf(a[s], v[s].z, mixv.z), mixv.w = fmaf(a[s], v[s].w, mixv.w);
+      }
+      u[k] = mixv;
+      ss += mixv.x * mixv.x + mixv.y * mixv.y + mixv.z * mixv.z + mixv.w * mixv.w;
+    }
+  }
+  if (!coeff) return;
+  ss = block_sum(ss, scratch);
+  const float rinv = 1.f / sqrtf(ss / (float)W + eps);
+#pragma unroll
+  for (int k = 0; k < KMAX; ++k) {
+    const int c = (threadIdx.x + k * 256) * 4;
+    if (c < W) {
+      if (sum_out) *reinterpret_cast<float4*>(sum_out + (size_t)i * W + c) = u[k];
+      if (out) {
+        T* op = out + (size_t)i * W + c;
+        op[0] = from_f<T>(u[k].x * rinv * to_f(w[c])), op[1] = from_f<T>(u[k].y * rinv * to_f(w[c + 1]));
+        op[2] = from_f<T>(u[k].z * rinv * to_f(w[c + 2])), op[3] = from_f<T>(u[k].w * rinv * to_f(w[c + 3]));
+      }
+    }
+  }
+}
+
+template <typename T, int S>
+static void stream_step_launch(float* x, const float* mix, const float* gain, const void* y, int y_stride, const float* coeff, const void* w,
+                               const int* rows, void* out, float* sum_out, int n, int W, float eps, int store, hipStream_t stream) {
+  if (W <= 2048)
+    stream_step_kernel<T, S, 2><<<n, 256, 0, stream>>>(x, mix, gain, (const T*)y, y_stride, coeff, (const T*)w, rows, (T*)out, sum_out, W, eps, store);
+  else
+    stream_step_kernel<T, S, 8><<<n, 256, 0, stream>>>(x, mix, gain, (const T*)y, y_stride, coeff, (const T*)w, rows, (T*)out, sum_out, W, eps, store);
+}
+
+extern "C" int ns_stream_step(float* x, const float* mix, const float* gain, const void* y, int y_stride, const float* coeff, const void* w,
+                              const int* rows, void* out, float* sum_out, int n, int S, int W, float eps, int store, int dtype,
+                              hipStream_t stream) {
+  if (n <= 0 || S <= 0 || S > 4 || W <= 0 || W > 8192 || W % 4 || (!y && !coeff)) return NS_ERR_BAD_ARG;
+  if (y && (!mix || !gain)) return NS_ERR_BAD_ARG;
+  if (y && rows && store) return NS_ERR_BAD_ARG;  // a write that is kept covers every row
+  if (dtype != NS_DTYPE_F32 && dtype != NS_DTYPE_BF16) return NS_ERR_UNSUPPORTED;
+#define NS_STEP(SS)                                                                                                                  \
+  if (dtype == NS_DTYPE_F32) stream_step_launch<float, SS>(x, mix, gain, y, y_stride, coeff, w, rows, out, sum_out, n, W, eps, store, stream); \
+  else stream_step_launch<bf16_t, SS>(x, mix, gain, y, y_stride, coeff, w, rows, out, sum_out, n, W, eps, store, stream)
+  switch (S) {
+    case 1: NS_STEP(1); break;
+    case 2: NS_STEP(2); break;
+    case 3: NS_STEP(3); break;
+    default: NS_STEP(4); break;
+  }
+#undef NS_STEP
+  return ns_launch_status();
+}
+
 // out = act(x), element by element; act 0: the tanh form of GELU, 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))); 1: SiLU
 template <typename T>
 __global__ void activation_kernel(T* __restrict__ out, const T* __restrict__ x, size_t count, int act) {
@@ -122,15 +228,45 @@ __global__ void activation_kernel(T* __restrict__ out, const T* __restrict__ x, 
   }
 }
 
+__device__ __forceinline__ float act_of(float z, int act) {
+  return act == 0 ? 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))) : z / (1.f + expf(-z));
+}
+
+// The same with 16-byte accesses, for counts that are a multiple of 16 bytes' worth and aligned pointers.
+template <typename T>
+__global__ void activation_vec_kernel(T* __restrict__ out, const T* __restrict__ x, size_t nvec, int act) {
+  constexpr int V = 16 / sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  const vec_t* xv = reinterpret_cast<const vec_t*>(x);
+  vec_t* ov = reinterpret_cast<vec_t*>(out);
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += (size_t)gridDim.x * blockDim.x) {
+    const vec_t a = xv[i];
+    vec_t r;
+#pragma unroll
+    for (int e = 0; e < V; ++e) r[e] = from_f<T>(act_of(to_f(a[e]), act));
+    ov[i] = r;
+  }
+}
+
 extern "C" int ns_activation(void* out, const void* x, size_t count, int act, int dtype, hipStream_t stream) {
   if (count == 0 || act < 0 || act > 1) return NS_ERR_BAD_ARG;
+  if (dtype != NS_DTYPE_F32 && dtype != NS_DTYPE_BF16) return NS_ERR_UNSUPPORTED;
+  const size_t per = dtype == NS_DTYPE_F32 ? 4 : 8;
+  if (count % per == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)x % 16) == 0) {
+    const size_t nvec = count / per;
+    size_t blocks = (nvec + 255) / 256;
+    if (blocks > 16384) blocks = 16384;
+    if (dtype == NS_DTYPE_F32)
+      activation_vec_kernel<float><<<(int)blocks, 256, 0, stream>>>((float*)out, (const float*)x, nvec, act);
+    else
+      activation_vec_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, nvec, act);
+    return ns_launch_status();
+  }
   size_t blocks = (count + 255) / 256;
   if (blocks > 65535) blocks = 65535;
   if (dtype == NS_DTYPE_F32)
     activation_kernel<float><<<(int)blocks, 256, 0, stream>>>((float*)out, (const float*)x, count, act);
-  else if (dtype == NS_DTYPE_BF16)
-    activation_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, count, act);
   else
-    return NS_ERR_UNSUPPORTED;
+    activation_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, count, act);
   return ns_launch_status();
 }

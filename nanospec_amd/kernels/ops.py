@@ -822,6 +822,64 @@ def stream_write(x: torch.Tensor, mix: torch.Tensor, gain: torch.Tensor, y: torc
                                         c_int(x.shape[2]), c_int(_dtype_code(y)), _stream()), "stream_write")
 
 
+STEP_MAX_STREAMS, STEP_MAX_WIDTH = 4, 8192  # what the one-pass kernel of ``stream_step`` takes (rows of a multiple of four columns)
+
+
+class PendingWrite:
+    """A sublayer's output on its way into a 32-bit stream: x_t <- sum_s mix[s, t] x_s + gain[t] * y, not done yet.
+    ``stream_step`` does it in the same pass as the next read."""
+
+    def __init__(self, y: torch.Tensor, mix: torch.Tensor, gain: torch.Tensor) -> None:
+        self.y, self.mix, self.gain = y, mix, gain
+
+
+def stream_step(x: torch.Tensor, pending: "PendingWrite | None", coeff: torch.Tensor | None = None, weight: torch.Tensor | None = None,
+                eps: float = 0.0, rows: torch.Tensor | None = None, out: torch.Tensor | None = None, sum_out: torch.Tensor | None = None,
+                store: bool = True) -> torch.Tensor | None:
+    """``stream_write`` of ``pending`` (if any) and then ``stream_read_norm`` with ``coeff`` and ``weight`` (if any), in one
+    pass over the rows where the sizes allow it, in two kernels otherwise.  With ``rows`` the read is of those rows only,
+    and a pending write is then done on the fly for them and not kept (``store`` must be False): for the last read of a step."""
+    S, W = x.shape[1], x.shape[2]
+    if pending is not None and rows is not None and store:
+        raise KernelRefused("stream_step: a write that is kept covers every row")
+    one_pass = S <= STEP_MAX_STREAMS and W <= STEP_MAX_WIDTH and W % 4 == 0
+    if not one_pass:
+        if pending is not None:  # (kept whatever ``store`` says: keeping it harms nobody)
+            stream_write(x, pending.mix, pending.gain, pending.y)
+        return stream_read_norm(x, coeff, weight, eps, rows=rows, out=out, sum_out=sum_out) if coeff is not None else None
+    _f32(x, "x")
+    y = None
+    if pending is not None:
+        y = pending.y
+        _f32(pending.mix, "mix"), _f32(pending.gain, "gain")
+        _gpu(y)
+        if pending.mix.shape != (S, S) or pending.gain.shape != (S,) or y.dim() != 2 or y.shape != (x.shape[0], W) or y.stride(1) != 1:
+            raise KernelRefused("stream_step: mix [S, S], gain [S], y [tokens, W]")
+    dtype = y.dtype if y is not None else weight.dtype
+    n = x.shape[0]
+    if coeff is not None:
+        _f32(coeff, "coeff")
+        _gpu(weight, rows, out, sum_out)
+        if coeff.numel() != S or weight.shape != (W,) or not weight.is_contiguous() or weight.dtype != dtype:
+            raise KernelRefused("stream_step: coeff [S], weight [W] in the dtype of y")
+        if rows is not None:
+            _i32(rows, "rows")
+            n = rows.numel()
+        if out is None:
+            out = torch.empty((n, W), dtype=dtype, device=x.device)
+        if out.shape != (n, W) or out.dtype != dtype or not out.is_contiguous():
+            raise KernelRefused("stream_step: out must be contiguous [rows, W] of the weight's dtype")
+        if sum_out is not None and _f32(sum_out, "sum_out").shape != (n, W):
+            raise KernelRefused("stream_step: sum_out must be float32 [rows, W]")
+    elif pending is None:
+        return None
+    _check(build.core().ns_stream_step(_ptr(x), _ptr(pending.mix if pending else None), _ptr(pending.gain if pending else None), _ptr(y),
+                                       c_int(y.stride(0) if y is not None else 0), _ptr(coeff), _ptr(weight), _ptr(rows), _ptr(out),
+                                       _ptr(sum_out), c_int(n), c_int(S), c_int(W), c_float(eps), c_int(1 if store else 0),
+                                       c_int(BF16 if dtype == torch.bfloat16 else F32), _stream()), "stream_step")
+    return out
+
+
 def activation(x: torch.Tensor, kind: str, out: torch.Tensor | None = None) -> torch.Tensor:
     """out = act(x) element by element (in place by default); ``kind`` one of ``ACTIVATIONS``."""
     _gpu(x, out)

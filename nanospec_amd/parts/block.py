@@ -185,24 +185,31 @@ class StreamBlock:
         return min(limits) if limits else None
 
     def forward(self, ctx, resid, delta, cache, owns_cache, delta_out):
-        """``resid``: float32 [tokens, S, width], updated in place; ``delta`` and ``delta_out`` are not used (nothing is
-        ever left to be added)."""
+        """``resid``: float32 [tokens, S, width], updated in place.  ``delta``: None, or the ``ops.PendingWrite`` that the block
+        before left (its last sublayer's output, not yet in the streams): it is written by the kernel that reads for this
+        block's mixer.  ``delta_out``: None, or a buffer [tokens, width] in the model's dtype that outlives the block: the
+        last sublayer's output is then left there, unwritten, and returned as a ``PendingWrite``.  (``delta`` may lie in the
+        same buffer: it is used up before anything is put there.)"""
         n, S, W = resid.shape
         if S != self.copies:
             raise ValueError(f"the block is built for {self.copies} streams, the model carries {S}")
         mark = ctx.arena.mark()
         dtype = self.mixer_norm.weight.dtype
         a, mix, gain = self._hc[0]
-        h = self.mixer_norm.read_streams(ctx, resid, a, out=ctx.arena.take((n, W), dtype))
-        y = self.mixer.forward(ctx, h, cache, owns_cache, out=ctx.arena.take((n, W), dtype))
-        ops.stream_write(resid, mix, gain, y)
-        if self.ffn is not None:
+        h = self.mixer_norm.read_streams(ctx, resid, a, out=ctx.arena.take((n, W), dtype), pending=delta)
+        last = self.ffn is None
+        y = self.mixer.forward(ctx, h, cache, owns_cache, out=delta_out if last and delta_out is not None else ctx.arena.take((n, W), dtype))
+        pending = ops.PendingWrite(y, mix, gain)
+        if not last:
             a, mix, gain = self._hc[1]
-            h = self.ffn_norm.read_streams(ctx, resid, a, out=h)
-            y = self.ffn.forward(ctx, h, out=y)
-            ops.stream_write(resid, mix, gain, y)
+            h = self.ffn_norm.read_streams(ctx, resid, a, out=h, pending=pending)
+            y = self.ffn.forward(ctx, h, out=delta_out if delta_out is not None else y)
+            pending = ops.PendingWrite(y, mix, gain)
+        if delta_out is None:
+            ops.stream_step(resid, pending)
+            pending = None
         ctx.arena.release(mark)
-        return None
+        return pending
 
 
 registry.register("block", "streams", StreamBlock)

@@ -135,13 +135,18 @@ class DecoderModel:
             # copies of the stream in 32-bit, all equal to the embedding's output; blocks update them in place
             resid = ctx.arena.take((n, self.spec.streams, self.spec.hidden), torch.float32)
             ops.embed_streams(self.embed, ctx.token_ids, resid, scale=self.spec.embed_scale)
+            # a block leaves its last sublayer's output unwritten (``ops.PendingWrite``): the next read writes it in passing
+            pending = None
+            carry = ctx.arena.take((n, self.spec.hidden), self.dtype)
             for i, call in enumerate(self.spec.run_order):
-                self.layers[call.layer].forward(ctx, resid, None, caches[i], call.cache_from is None, None)
+                pending = self.layers[call.layer].forward(ctx, resid, pending, caches[i], call.cache_from is None, carry)
                 if self.layer_probe is not None:
                     total = torch.empty((n, self.spec.hidden), dtype=torch.float32, device=resid.device)
-                    self.final_norm.read_streams(ctx, resid, self._ones, out=ctx.arena.take((n, self.spec.hidden), self.dtype), sum_out=total)
+                    self.final_norm.read_streams(ctx, resid, self._ones, out=ctx.arena.take((n, self.spec.hidden), self.dtype), sum_out=total,
+                                                 pending=pending)
+                    pending = None
                     self.layer_probe(i, total)
-            return resid, None
+            return resid, pending
         resid = ctx.arena.take((n, self.spec.hidden), self.dtype)
         delta = ctx.arena.take((n, self.spec.hidden), self.dtype)
         ops.embed(self.embed, ctx.token_ids, out=resid, scale=self.spec.embed_scale)
@@ -171,7 +176,10 @@ class DecoderModel:
         (reference: model/llama.py:284-286, engine/engine.py:382)."""
         n = rows.numel()
         if self.spec.streams:  # the streams are added up as the last norm reads them
-            h = self.final_norm.read_streams(ctx, resid, self._ones, rows=rows, out=ctx.arena.take((n, self.spec.hidden), self.dtype))
+            # (what the last block left unwritten is added for these rows as they are read, and not kept: nobody reads the
+            # streams again)
+            h = self.final_norm.read_streams(ctx, resid, self._ones, rows=rows, out=ctx.arena.take((n, self.spec.hidden), self.dtype),
+                                             pending=delta, store=False)
         else:
             h = self.final_norm.forward(ctx, resid=resid, x=delta, rows=rows, out=ctx.arena.take((n, self.spec.hidden), self.dtype))
         out = self.head(h, out=ctx.arena.take((n, self.spec.vocab_size), torch.float32), out_f32=True, arena=ctx.arena)

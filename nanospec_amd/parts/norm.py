@@ -27,10 +27,13 @@ class RMSNorm:
     def forward(self, ctx, resid=None, x=None, rows=None, write_resid=False, out=None) -> torch.Tensor:
         return ops.rmsnorm(self.weight, self.spec.eps, resid=resid, x=x, rows=rows, write_resid=write_resid, out=out)
 
-    def read_streams(self, ctx, streams: torch.Tensor, coeff: torch.Tensor, rows=None, out=None, sum_out=None) -> torch.Tensor:
+    def read_streams(self, ctx, streams: torch.Tensor, coeff: torch.Tensor, rows=None, out=None, sum_out=None, pending=None,
+                     store: bool = True) -> torch.Tensor:
         """The norm of one mix of a 32-bit residual stream's copies: u = sum_s coeff[s] streams[:, s]; weight * u / rms(u),
-        in the weight's dtype (``streams`` float32 [tokens, S, dim]; see ``parts.block.StreamBlock``)."""
-        return ops.stream_read_norm(streams, coeff, self.weight, self.spec.eps, rows=rows, out=out, sum_out=sum_out)
+        in the weight's dtype (``streams`` float32 [tokens, S, dim]; see ``parts.block.StreamBlock``).  ``pending``: a
+        sublayer's output that is still to be written into the streams (``ops.PendingWrite``); it is written in the same
+        pass, before the read (with ``rows`` and ``store`` = False: for those rows only and without keeping it)."""
+        return ops.stream_step(streams, pending, coeff, self.weight, self.spec.eps, rows=rows, out=out, sum_out=sum_out, store=store)
 
 
 register("norm", "rmsnorm", RMSNorm)

@@ -292,6 +292,40 @@ def test_stream_read_and_write(S, W, dtype):
         torch.testing.assert_close(e[:, s].cpu(), table[ids.cpu().long()].float() * 1.5)
 
 
+@pytest.mark.parametrize("S,W", [(1, 64), (2, 96), (3, 2048), (4, 4100), (5, 96), (3, 90)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_stream_write_and_read_in_one_pass(S, W, dtype):
+    """A sublayer's output written and the next sublayer's input read by one kernel (and by two where the sizes are not the
+    one-pass kernel's), kept or, for a few rows at a step's end, not kept."""
+    from nanospec_amd.kernels import ops
+
+    torch.manual_seed(S * W)
+    n = 6
+    x = torch.randn(n, S, W)
+    a, mix, gain, w = torch.randn(S), torch.randn(S, S), torch.randn(S), (1 + 0.1 * torch.randn(W)).to(dtype)
+    y = torch.randn(n, W).to(dtype)
+    new = torch.einsum("st,nsw->ntw", mix.double(), x.double()) + gain.double().view(1, S, 1) * y.double().view(n, 1, W)
+    u = torch.einsum("s,nsw->nw", a.double(), new)
+    ref = pv.rms(u, 1e-5) * w.double()
+    tol = dict(rtol=1e-5, atol=1e-5) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-2)
+    pend = ops.PendingWrite(y.to(DEV), mix.to(DEV), gain.to(DEV))
+    xd = x.to(DEV)
+    h = ops.stream_step(xd, pend, a.to(DEV), w.to(DEV), 1e-5)
+    torch.testing.assert_close(h.cpu().double(), ref, **tol)
+    torch.testing.assert_close(xd.cpu().double(), new, rtol=1e-5, atol=1e-5)
+    xd = x.to(DEV)
+    rows = torch.tensor([4, 1], dtype=torch.int32, device=DEV)
+    total = torch.empty(2, W, device=DEV)
+    h = ops.stream_step(xd, pend, a.to(DEV), w.to(DEV), 1e-5, rows=rows, sum_out=total, store=False)
+    torch.testing.assert_close(h.cpu().double(), ref[[4, 1]], **tol)
+    torch.testing.assert_close(total.cpu().double(), u[[4, 1]], rtol=1e-5, atol=1e-5)
+    xd = x.to(DEV)
+    assert ops.stream_step(xd, pend) is None  # a write alone
+    torch.testing.assert_close(xd.cpu().double(), new, rtol=1e-5, atol=1e-5)
+    h = ops.stream_step(xd, None, a.to(DEV), w.to(DEV), 1e-5)  # a read alone
+    torch.testing.assert_close(h.cpu().double(), ref, **tol)
+
+
 def test_activation_is_the_tanh_form():
     from nanospec_amd.kernels import ops
 
