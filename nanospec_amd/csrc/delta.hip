@@ -131,18 +131,30 @@ extern "C" int ns_delta_prep(float* qkv, int C, float* g, float* beta, const voi
 // current stage's tokens are worked through from LDS, and then written to the other LDS buffer.  The arithmetic of a
 // token is the same whatever the stage it falls into: results do not depend on how a prompt was cut.
 // ------------------------------------------------------------------------------------------------
+// The sum of a value over the RG neighbouring lanes of a column, in all of them.  Up to 16 lanes lie in one row of the
+// wave, where a lane reads its partner through the data path of the vector unit itself (quad permutations, then the
+// mirrored half row and row: any partner in the other half will do for a sum); wider groups go on through LDS's crossbar.
+template <int CTRL>
+__device__ __forceinline__ float dpp_read(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
 __device__ __forceinline__ float group_sum(float v, int rg_count) {
-  for (int o = 1; o < rg_count; o <<= 1) v += __shfl_xor(v, o, NS_WAVE);
+  if (rg_count >= 2) v += dpp_read<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+  if (rg_count >= 4) v += dpp_read<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+  if (rg_count >= 8) v += dpp_read<0x141>(v);  // row_half_mirror
+  if (rg_count >= 16) v += dpp_read<0x140>(v); // row_mirror
+  for (int o = 16; o < rg_count; o <<= 1) v += __shfl_xor(v, o, NS_WAVE);
   return v;
 }
 
 #define ND_STAGE_FLOATS 6144                       // floats of one stage in LDS (two stages are held)
-#define ND_STAGE_REGS (ND_STAGE_FLOATS / 256)      // of which each of the 256 threads fetches this many
+#define ND_STAGE_REGS (ND_STAGE_FLOATS / 1024)     // of which each of the 256 threads fetches this many groups of four
 
 struct DeltaShape {
-  int C, H, G, D, E, RG, Dp, dp_shift, cols, tok_stride, stage_tokens;
+  int C, H, G, D, E, RG, Dp, dp_shift, cols, tok_stride, stage_tokens, vec4;
 };
 
+template <bool VEC>
 __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, const float* __restrict__ qkv,
                                                          const float* __restrict__ g, const float* __restrict__ beta,
                                                          float* __restrict__ state, size_t slot_stride, const int* __restrict__ qo_indptr,
@@ -168,39 +180,53 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
   const float* v_src = qkv + (size_t)2 * p.G * D + (size_t)h * E + j0;
   const float* g_src = g + (size_t)h * D;
   const int stage_elems = p.stage_tokens * p.tok_stride;
-  auto fetch = [&](float (&regs)[ND_STAGE_REGS], int first) {
-    int tt = threadIdx.x / p.tok_stride, off = threadIdx.x - tt * p.tok_stride;  // of element e, kept up as e grows by 256
+  // A thread fetches groups of four floats; every part of a token's record starts at a multiple of four.  The loads are
+  // issued without a branch around any of them (addresses of groups that hold nothing are bent to the start of the
+  // source and their values dropped), so that all of a stage's loads are in flight together.
+  // (what is kept of a loaded group is decided when it is parked, so that nothing here waits for a load)
+  struct Stage {
+    float4 v[ND_STAGE_REGS];
+    float bt[ND_STAGE_REGS];
+    unsigned keep, is_beta;  // four bits a group: which of its floats are kept; one bit a group: its first float is beta
+  };
+  auto fetch = [&](Stage& st, int first) {
+    int tt = threadIdx.x * 4 / p.tok_stride, off = threadIdx.x * 4 - tt * p.tok_stride;  // of element e, kept up as e grows by 1024
+    st.keep = st.is_beta = 0;
 #pragma unroll
     for (int i = 0; i < ND_STAGE_REGS; ++i) {
-      const int e = threadIdx.x + i * 256;
-      float val = 0.f;
-      if (e < stage_elems) {
-        const int r = first + tt;
-        if (r < r1) {
-          const int part = off >> p.dp_shift, d = off & (p.Dp - 1);
-          if (part < 3) {
-            if (d < D) val = part == 0 ? q_src[(size_t)r * p.C + d] : (part == 1 ? k_src[(size_t)r * p.C + d] : g_src[(size_t)r * p.H * D + d]);
-          } else {
-            const int c = off - 3 * p.Dp;
-            if (c < p.cols) val = j0 + c < E ? v_src[(size_t)r * p.C + c] : 0.f;
-            else if (c == p.cols) val = beta[(size_t)r * p.H + h];
-          }
-        }
+      const int e = (threadIdx.x + i * 256) * 4;
+      const int r = min(first + tt, r1 - 1);
+      const bool live = e < stage_elems && first + tt < r1;
+      const int part = off >> p.dp_shift, d = off & (p.Dp - 1);
+      const int c = off - 3 * p.Dp;
+      const float* src = part == 0 ? q_src + (size_t)r * p.C : (part == 1 ? k_src + (size_t)r * p.C : (part == 2 ? g_src + (size_t)r * p.H * D : v_src + (size_t)r * p.C));
+      const int at = part < 3 ? d : c;
+      const int lim = !live ? 0 : (part < 3 ? D : min(p.cols, E - j0));
+      if constexpr (VEC) {
+        st.v[i] = *reinterpret_cast<const float4*>(src + (at < lim ? at : 0));
+        st.keep |= (at < lim ? 0xfu : 0u) << (4 * i);
+      } else {
+        st.v[i] = float4{src[at < lim ? at : 0], src[at + 1 < lim ? at + 1 : 0], src[at + 2 < lim ? at + 2 : 0], src[at + 3 < lim ? at + 3 : 0]};
+        st.keep |= ((at < lim ? 1u : 0u) | (at + 1 < lim ? 2u : 0u) | (at + 2 < lim ? 4u : 0u) | (at + 3 < lim ? 8u : 0u)) << (4 * i);
       }
-      regs[i] = val;
-      off += 256;
+      st.bt[i] = beta[(size_t)r * p.H + h];
+      st.is_beta |= (live && part >= 3 && c == p.cols ? 1u : 0u) << i;
+      off += 1024;
       while (off >= p.tok_stride) off -= p.tok_stride, ++tt;
     }
   };
-  auto park = [&](const float (&regs)[ND_STAGE_REGS], float* buf) {
+  auto park = [&](const Stage& st, float* buf) {
 #pragma unroll
     for (int i = 0; i < ND_STAGE_REGS; ++i) {
-      const int e = threadIdx.x + i * 256;
-      if (e < stage_elems) buf[e] = regs[i];
+      const int e = (threadIdx.x + i * 256) * 4;
+      const unsigned k = st.keep >> (4 * i);
+      float4 val = {k & 1u ? st.v[i].x : 0.f, k & 2u ? st.v[i].y : 0.f, k & 4u ? st.v[i].z : 0.f, k & 8u ? st.v[i].w : 0.f};
+      if ((st.is_beta >> i) & 1u) val.x = st.bt[i];
+      if (e < stage_elems) *reinterpret_cast<float4*>(buf + e) = val;
     }
   };
 
-  float regs[ND_STAGE_REGS];
+  Stage regs;
   fetch(regs, r0);
   park(regs, stage[0]);
   __syncthreads();
@@ -210,38 +236,49 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
     if (more) fetch(regs, first + p.stage_tokens);
     const float* buf = stage[cur];
     const int n = min(p.stage_tokens, r1 - first);
-    for (int tt = 0; tt < n; ++tt) {
+    // the next token's operands are read from LDS while this token's chain runs
+    float4 qn[ND_ROWS / 4], kn[ND_ROWS / 4], gn[ND_ROWS / 4];
+    float vn, bn;
+    auto read_token = [&](int tt) {
       const float* tok = buf + tt * p.tok_stride;
-      const float4* q4 = reinterpret_cast<const float4*>(tok + d0);
-      const float4* k4 = reinterpret_cast<const float4*>(tok + p.Dp + d0);
-      const float4* g4 = reinterpret_cast<const float4*>(tok + 2 * p.Dp + d0);
-      const float vc = tok[3 * p.Dp + jl], bc = tok[3 * p.Dp + p.cols];
-      float kk[ND_ROWS];
-      float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i = 0; i < ND_ROWS / 4; ++i) {
-        const float4 gv = g4[i], kv = k4[i];
+        qn[i] = reinterpret_cast<const float4*>(tok + d0)[i];
+        kn[i] = reinterpret_cast<const float4*>(tok + p.Dp + d0)[i];
+        gn[i] = reinterpret_cast<const float4*>(tok + 2 * p.Dp + d0)[i];
+      }
+      vn = tok[3 * p.Dp + jl], bn = tok[3 * p.Dp + p.cols];
+    };
+    read_token(0);
+    for (int tt = 0; tt < n; ++tt) {
+      float kk[ND_ROWS], qq[ND_ROWS];
+      float part[4] = {0.f, 0.f, 0.f, 0.f};
+      const float vc = vn, bc = bn;
+#pragma unroll
+      for (int i = 0; i < ND_ROWS / 4; ++i) {
+        const float4 gv = gn[i], kv = kn[i], qv = qn[i];
         kk[4 * i] = kv.x, kk[4 * i + 1] = kv.y, kk[4 * i + 2] = kv.z, kk[4 * i + 3] = kv.w;
+        qq[4 * i] = qv.x, qq[4 * i + 1] = qv.y, qq[4 * i + 2] = qv.z, qq[4 * i + 3] = qv.w;
         s[4 * i] *= gv.x, s[4 * i + 1] *= gv.y, s[4 * i + 2] *= gv.z, s[4 * i + 3] *= gv.w;
         part[0] = fmaf(kv.x, s[4 * i], part[0]);
         part[1] = fmaf(kv.y, s[4 * i + 1], part[1]);
         part[2] = fmaf(kv.z, s[4 * i + 2], part[2]);
         part[3] = fmaf(kv.w, s[4 * i + 3], part[3]);
       }
+      if (tt + 1 < n) read_token(tt + 1);
       const float dot = group_sum((part[0] + part[1]) + (part[2] + part[3]), RG);
       const float u = bc * (vc - dot);
       float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i = 0; i < ND_ROWS / 4; ++i) {
-        const float4 qv = q4[i];
         s[4 * i] = fmaf(kk[4 * i], u, s[4 * i]);
         s[4 * i + 1] = fmaf(kk[4 * i + 1], u, s[4 * i + 1]);
         s[4 * i + 2] = fmaf(kk[4 * i + 2], u, s[4 * i + 2]);
         s[4 * i + 3] = fmaf(kk[4 * i + 3], u, s[4 * i + 3]);
-        acc[0] = fmaf(qv.x, s[4 * i], acc[0]);
-        acc[1] = fmaf(qv.y, s[4 * i + 1], acc[1]);
-        acc[2] = fmaf(qv.z, s[4 * i + 2], acc[2]);
-        acc[3] = fmaf(qv.w, s[4 * i + 3], acc[3]);
+        acc[0] = fmaf(qq[4 * i], s[4 * i], acc[0]);
+        acc[1] = fmaf(qq[4 * i + 1], s[4 * i + 1], acc[1]);
+        acc[2] = fmaf(qq[4 * i + 2], s[4 * i + 2], acc[2]);
+        acc[3] = fmaf(qq[4 * i + 3], s[4 * i + 3], acc[3]);
       }
       const float out = group_sum((acc[0] + acc[1]) + (acc[2] + acc[3]), RG);
       if (rg == 0 && col_ok) o[(size_t)(first + tt) * p.H * E + (size_t)h * E + j] = out;
@@ -270,9 +307,14 @@ extern "C" int ns_delta_scan(float* o, const float* qkv, int C, const float* g, 
   p.stage_tokens = ND_STAGE_FLOATS / p.tok_stride;
   if (p.stage_tokens < 1) return NS_ERR_BAD_ARG;
   if (p.stage_tokens > 64) p.stage_tokens = 64;
+  // 16-byte loads where every group of four that a thread fetches starts at a multiple of four floats
+  p.vec4 = (D % 4 == 0 && E % 4 == 0 && C % 4 == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)g % 16) == 0) ? 1 : 0;
   const int zb = (E + p.cols - 1) / p.cols;
   if (zb > 65535) return NS_ERR_BAD_ARG;
-  delta_scan_kernel<<<dim3(n_reqs, H, zb), 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p);
+  if (p.vec4)
+    delta_scan_kernel<true><<<dim3(n_reqs, H, zb), 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p);
+  else
+    delta_scan_kernel<false><<<dim3(n_reqs, H, zb), 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p);
   return ns_launch_status();
 }
 
