@@ -138,23 +138,26 @@ template <int CTRL>
 __device__ __forceinline__ float dpp_read(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
-__device__ __forceinline__ float group_sum(float v, int rg_count) {
-  if (rg_count >= 2) v += dpp_read<0xB1>(v);   // quad_perm [1, 0, 3, 2]
-  if (rg_count >= 4) v += dpp_read<0x4E>(v);   // quad_perm [2, 3, 0, 1]
-  if (rg_count >= 8) v += dpp_read<0x141>(v);  // row_half_mirror
-  if (rg_count >= 16) v += dpp_read<0x140>(v); // row_mirror
-  for (int o = 16; o < rg_count; o <<= 1) v += __shfl_xor(v, o, NS_WAVE);
+template <int RGC>
+__device__ __forceinline__ float group_sum(float v) {
+  if constexpr (RGC >= 2) v += dpp_read<0xB1>(v);   // quad_perm [1, 0, 3, 2]
+  if constexpr (RGC >= 4) v += dpp_read<0x4E>(v);   // quad_perm [2, 3, 0, 1]
+  if constexpr (RGC >= 8) v += dpp_read<0x141>(v);  // row_half_mirror
+  if constexpr (RGC >= 16) v += dpp_read<0x140>(v); // row_mirror
+#pragma unroll
+  for (int o = 16; o < RGC; o <<= 1) v += __shfl_xor(v, o, NS_WAVE);
   return v;
 }
 
+#define ND_PITCH (ND_ROWS + 4)                     // floats between two row groups' channels in LDS
 #define ND_STAGE_FLOATS 6144                       // floats of one stage in LDS (two stages are held)
 #define ND_STAGE_REGS (ND_STAGE_FLOATS / 1024)     // of which each of the 256 threads fetches this many groups of four
 
 struct DeltaShape {
-  int C, H, G, D, E, RG, Dp, dp_shift, cols, tok_stride, stage_tokens, vec4;
+  int C, H, G, D, E, RG, Dl, cols, tok_stride, stage_tokens, vec4;
 };
 
-template <bool VEC>
+template <bool VEC, int RG>
 __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, const float* __restrict__ qkv,
                                                          const float* __restrict__ g, const float* __restrict__ beta,
                                                          float* __restrict__ state, size_t slot_stride, const int* __restrict__ qo_indptr,
@@ -163,9 +166,10 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
   const int b = blockIdx.x, h = blockIdx.y;
   const int r0 = qo_indptr[b], r1 = qo_indptr[b + 1];
   if (r1 <= r0) return;
-  const int D = p.D, E = p.E, RG = p.RG;
+  const int D = p.D, E = p.E;
+  constexpr int DL = RG * ND_PITCH, COLS = 256 / RG;
   const int jl = threadIdx.x / RG, rg = threadIdx.x % RG;
-  const int j0 = blockIdx.z * p.cols, j = j0 + jl;
+  const int j0 = blockIdx.z * COLS, j = j0 + jl;
   const bool col_ok = j < E;
   const int d0 = rg * ND_ROWS;
   const int kh = h / (p.H / p.G);
@@ -174,7 +178,9 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
 #pragma unroll
   for (int i = 0; i < ND_ROWS; ++i) s[i] = (col_ok && d0 + i < D) ? S[(size_t)(d0 + i) * E + j] : 0.f;
 
-  // what element e of a stage that starts at row `first` is: token e / tok_stride, then q [Dp] | k [Dp] | g [Dp] | v [cols] | beta
+  // what element e of a stage that starts at row `first` is: token e / tok_stride, then q [Dl] | k [Dl] | g [Dl] | v [cols] | beta;
+  // in q, k and g the 16 channels of a row group are followed by four unused floats (ND_PITCH), so that the row groups'
+  // 16-byte reads fall into different banks
   const float* q_src = qkv + (size_t)kh * D;
   const float* k_src = qkv + (size_t)p.G * D + (size_t)kh * D;
   const float* v_src = qkv + (size_t)2 * p.G * D + (size_t)h * E + j0;
@@ -197,11 +203,13 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
       const int e = (threadIdx.x + i * 256) * 4;
       const int r = min(first + tt, r1 - 1);
       const bool live = e < stage_elems && first + tt < r1;
-      const int part = off >> p.dp_shift, d = off & (p.Dp - 1);
-      const int c = off - 3 * p.Dp;
+      const int part = off < DL ? 0 : (off < 2 * DL ? 1 : (off < 3 * DL ? 2 : 3));
+      const int within = off - part * DL, chunk = within / ND_PITCH, w = within - chunk * ND_PITCH;
+      const int d = w < ND_ROWS ? chunk * ND_ROWS + w : 0x3fffffff;  // (the unused floats keep nothing)
+      const int c = off - 3 * DL;
       const float* src = part == 0 ? q_src + (size_t)r * p.C : (part == 1 ? k_src + (size_t)r * p.C : (part == 2 ? g_src + (size_t)r * p.H * D : v_src + (size_t)r * p.C));
       const int at = part < 3 ? d : c;
-      const int lim = !live ? 0 : (part < 3 ? D : min(p.cols, E - j0));
+      const int lim = !live ? 0 : (part < 3 ? D : min(COLS, E - j0));
       if constexpr (VEC) {
         st.v[i] = *reinterpret_cast<const float4*>(src + (at < lim ? at : 0));
         st.keep |= (at < lim ? 0xfu : 0u) << (4 * i);
@@ -210,7 +218,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
         st.keep |= ((at < lim ? 1u : 0u) | (at + 1 < lim ? 2u : 0u) | (at + 2 < lim ? 4u : 0u) | (at + 3 < lim ? 8u : 0u)) << (4 * i);
       }
       st.bt[i] = beta[(size_t)r * p.H + h];
-      st.is_beta |= (live && part >= 3 && c == p.cols ? 1u : 0u) << i;
+      st.is_beta |= (live && part >= 3 && c == COLS ? 1u : 0u) << i;
       off += 1024;
       while (off >= p.tok_stride) off -= p.tok_stride, ++tt;
     }
@@ -226,6 +234,10 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
     }
   };
 
+  // where this thread's output of the next token goes (the first lane of a column's group writes it)
+  const bool writes = rg == 0 && col_ok;
+  const size_t out_stride = (size_t)p.H * E;
+  float* op = o + (size_t)r0 * out_stride + (size_t)h * E + (col_ok ? j : 0);
   Stage regs;
   fetch(regs, r0);
   park(regs, stage[0]);
@@ -236,52 +248,59 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
     if (more) fetch(regs, first + p.stage_tokens);
     const float* buf = stage[cur];
     const int n = min(p.stage_tokens, r1 - first);
-    // the next token's operands are read from LDS while this token's chain runs
-    float4 qn[ND_ROWS / 4], kn[ND_ROWS / 4], gn[ND_ROWS / 4];
-    float vn, bn;
-    auto read_token = [&](int tt) {
+    // Two sets of operand registers take turns: the next token's operands are read from LDS into one while the chain of
+    // the current token runs on the other (written out twice, so that no set is ever copied into the other).
+    struct Operands {
+      float4 q[ND_ROWS / 4], k[ND_ROWS / 4], g[ND_ROWS / 4];
+      float v, b;
+    };
+    auto read_token = [&](Operands& t, int tt) {
       const float* tok = buf + tt * p.tok_stride;
 #pragma unroll
       for (int i = 0; i < ND_ROWS / 4; ++i) {
-        qn[i] = reinterpret_cast<const float4*>(tok + d0)[i];
-        kn[i] = reinterpret_cast<const float4*>(tok + p.Dp + d0)[i];
-        gn[i] = reinterpret_cast<const float4*>(tok + 2 * p.Dp + d0)[i];
+        t.q[i] = reinterpret_cast<const float4*>(tok + rg * ND_PITCH)[i];
+        t.k[i] = reinterpret_cast<const float4*>(tok + DL + rg * ND_PITCH)[i];
+        t.g[i] = reinterpret_cast<const float4*>(tok + 2 * DL + rg * ND_PITCH)[i];
       }
-      vn = tok[3 * p.Dp + jl], bn = tok[3 * p.Dp + p.cols];
+      t.v = tok[3 * DL + jl], t.b = tok[3 * DL + COLS];
     };
-    read_token(0);
-    for (int tt = 0; tt < n; ++tt) {
-      float kk[ND_ROWS], qq[ND_ROWS];
+    auto chain = [&](const Operands& t) {
       float part[4] = {0.f, 0.f, 0.f, 0.f};
-      const float vc = vn, bc = bn;
 #pragma unroll
       for (int i = 0; i < ND_ROWS / 4; ++i) {
-        const float4 gv = gn[i], kv = kn[i], qv = qn[i];
-        kk[4 * i] = kv.x, kk[4 * i + 1] = kv.y, kk[4 * i + 2] = kv.z, kk[4 * i + 3] = kv.w;
-        qq[4 * i] = qv.x, qq[4 * i + 1] = qv.y, qq[4 * i + 2] = qv.z, qq[4 * i + 3] = qv.w;
-        s[4 * i] *= gv.x, s[4 * i + 1] *= gv.y, s[4 * i + 2] *= gv.z, s[4 * i + 3] *= gv.w;
-        part[0] = fmaf(kv.x, s[4 * i], part[0]);
-        part[1] = fmaf(kv.y, s[4 * i + 1], part[1]);
-        part[2] = fmaf(kv.z, s[4 * i + 2], part[2]);
-        part[3] = fmaf(kv.w, s[4 * i + 3], part[3]);
+        s[4 * i] *= t.g[i].x, s[4 * i + 1] *= t.g[i].y, s[4 * i + 2] *= t.g[i].z, s[4 * i + 3] *= t.g[i].w;
+        part[0] = fmaf(t.k[i].x, s[4 * i], part[0]);
+        part[1] = fmaf(t.k[i].y, s[4 * i + 1], part[1]);
+        part[2] = fmaf(t.k[i].z, s[4 * i + 2], part[2]);
+        part[3] = fmaf(t.k[i].w, s[4 * i + 3], part[3]);
       }
-      if (tt + 1 < n) read_token(tt + 1);
-      const float dot = group_sum((part[0] + part[1]) + (part[2] + part[3]), RG);
-      const float u = bc * (vc - dot);
+      const float dot = group_sum<RG>((part[0] + part[1]) + (part[2] + part[3]));
+      const float u = t.b * (t.v - dot);
       float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int i = 0; i < ND_ROWS / 4; ++i) {
-        s[4 * i] = fmaf(kk[4 * i], u, s[4 * i]);
-        s[4 * i + 1] = fmaf(kk[4 * i + 1], u, s[4 * i + 1]);
-        s[4 * i + 2] = fmaf(kk[4 * i + 2], u, s[4 * i + 2]);
-        s[4 * i + 3] = fmaf(kk[4 * i + 3], u, s[4 * i + 3]);
-        acc[0] = fmaf(qq[4 * i], s[4 * i], acc[0]);
-        acc[1] = fmaf(qq[4 * i + 1], s[4 * i + 1], acc[1]);
-        acc[2] = fmaf(qq[4 * i + 2], s[4 * i + 2], acc[2]);
-        acc[3] = fmaf(qq[4 * i + 3], s[4 * i + 3], acc[3]);
+        s[4 * i] = fmaf(t.k[i].x, u, s[4 * i]);
+        s[4 * i + 1] = fmaf(t.k[i].y, u, s[4 * i + 1]);
+        s[4 * i + 2] = fmaf(t.k[i].z, u, s[4 * i + 2]);
+        s[4 * i + 3] = fmaf(t.k[i].w, u, s[4 * i + 3]);
+        acc[0] = fmaf(t.q[i].x, s[4 * i], acc[0]);
+        acc[1] = fmaf(t.q[i].y, s[4 * i + 1], acc[1]);
+        acc[2] = fmaf(t.q[i].z, s[4 * i + 2], acc[2]);
+        acc[3] = fmaf(t.q[i].w, s[4 * i + 3], acc[3]);
       }
-      const float out = group_sum((acc[0] + acc[1]) + (acc[2] + acc[3]), RG);
-      if (rg == 0 && col_ok) o[(size_t)(first + tt) * p.H * E + (size_t)h * E + j] = out;
+      const float out = group_sum<RG>((acc[0] + acc[1]) + (acc[2] + acc[3]));
+      if (writes) *op = out;
+      op += out_stride;
+    };
+    Operands ta, tb;
+    read_token(ta, 0);
+    for (int tt = 0; tt < n; tt += 2) {
+      if (tt + 1 < n) read_token(tb, tt + 1);
+      chain(ta);
+      if (tt + 1 < n) {
+        if (tt + 2 < n) read_token(ta, tt + 2);
+        chain(tb);
+      }
     }
     if (more) park(regs, stage[cur ^ 1]);
     __syncthreads();
@@ -299,11 +318,9 @@ extern "C" int ns_delta_scan(float* o, const float* qkv, int C, const float* g, 
   p.C = C, p.H = H, p.G = G, p.D = D, p.E = E;
   p.RG = 1;
   while (p.RG * ND_ROWS < D) p.RG *= 2;
-  p.Dp = p.RG * ND_ROWS;
-  p.dp_shift = 0;
-  while ((1 << p.dp_shift) < p.Dp) ++p.dp_shift;
+  p.Dl = p.RG * ND_PITCH;
   p.cols = 256 / p.RG;
-  p.tok_stride = 3 * p.Dp + ((p.cols + 1 + 3) / 4) * 4;
+  p.tok_stride = 3 * p.Dl + ((p.cols + 1 + 3) / 4) * 4;
   p.stage_tokens = ND_STAGE_FLOATS / p.tok_stride;
   if (p.stage_tokens < 1) return NS_ERR_BAD_ARG;
   if (p.stage_tokens > 64) p.stage_tokens = 64;
@@ -311,10 +328,22 @@ extern "C" int ns_delta_scan(float* o, const float* qkv, int C, const float* g, 
   p.vec4 = (D % 4 == 0 && E % 4 == 0 && C % 4 == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)g % 16) == 0) ? 1 : 0;
   const int zb = (E + p.cols - 1) / p.cols;
   if (zb > 65535) return NS_ERR_BAD_ARG;
-  if (p.vec4)
-    delta_scan_kernel<true><<<dim3(n_reqs, H, zb), 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p);
-  else
-    delta_scan_kernel<false><<<dim3(n_reqs, H, zb), 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p);
+  const dim3 grid(n_reqs, H, zb);
+#define ND_LAUNCH(R)                                                                                                             \
+  case R:                                                                                                                         \
+    if (p.vec4) delta_scan_kernel<true, R><<<grid, 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p); \
+    else delta_scan_kernel<false, R><<<grid, 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p);       \
+    break
+  switch (p.RG) {
+    ND_LAUNCH(1);
+    ND_LAUNCH(2);
+    ND_LAUNCH(4);
+    ND_LAUNCH(8);
+    ND_LAUNCH(16);
+    ND_LAUNCH(32);
+    default: ND_LAUNCH(64);
+  }
+#undef ND_LAUNCH
   return ns_launch_status();
 }
 
