@@ -231,7 +231,7 @@ def vuzelix_config(shape: dict, layers: int | None = None):
 
 def design_compare(a) -> int:
     """``--design vuzelix``: prefill and decode throughput of the Vuzelix design beside the Llama model of the same shape,
-    one JSON line.  The default workload and its contract are not touched by this option."""
+    one JSON line.  The default workload and its output are not touched by this option."""
     import types
 
     import torch

@@ -97,17 +97,19 @@ extern "C" int ns_attn_generic(void* out, const void* q, int q_stride, const voi
 // queries in place; keys and values go into the pages of their positions.  A row of ``qkv`` is q [heads][hd], then, if
 // the layer has keys and values of its own (``own_kv``), k [kv_heads][hd] and v [kv_heads][vd].
 // ------------------------------------------------------------------------------------------------
+// grid (tokens, Y): a wave takes one head's vector; the blocks after those copy the values, 1,024 a block.
 template <typename T>
 __global__ void unit_kv_write_kernel(T* __restrict__ qkv, int stride, const int* __restrict__ positions, const int* __restrict__ token_req,
                                      const int* __restrict__ block_table, int table_stride, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                     int heads, int kv_heads, int hd, int vd, int page_size, float eps, int own_kv) {
-  const int t = blockIdx.x, lane = threadIdx.x & (NS_WAVE - 1), wave = threadIdx.x / NS_WAVE, nw = blockDim.x / NS_WAVE;
+                                     int heads, int kv_heads, int hd, int vd, int page_size, float eps, int own_kv, int vec_blocks) {
+  const int t = blockIdx.x, lane = threadIdx.x & (NS_WAVE - 1), wave = threadIdx.x / NS_WAVE;
   T* row = qkv + (size_t)t * stride;
   const int pos = positions[t];
   const int page = own_kv ? block_table[(size_t)token_req[t] * table_stride + pos / page_size] : 0;
   const int slot = pos % page_size;
-  const int vecs = heads + (own_kv ? kv_heads : 0);
-  for (int vec = wave; vec < vecs; vec += nw) {
+  if ((int)blockIdx.y < vec_blocks) {
+    const int vec = blockIdx.y * 4 + wave;
+    if (vec >= heads + (own_kv ? kv_heads : 0)) return;
     T* p = row + (size_t)vec * hd;
     float f = 1.f;
     if (eps >= 0.f) {
@@ -123,10 +125,12 @@ __global__ void unit_kv_write_kernel(T* __restrict__ qkv, int stride, const int*
       T* dst = k_cache + (((size_t)page * kv_heads + (vec - heads)) * page_size + slot) * hd;
       for (int d = lane; d < hd; d += NS_WAVE) dst[d] = from_f<T>(to_f(p[d]) * f);
     }
+    return;
   }
   if (own_kv) {
     const T* v = row + (size_t)(heads + kv_heads) * hd;
-    for (int i = threadIdx.x; i < kv_heads * vd; i += blockDim.x)
+    const int part = blockIdx.y - vec_blocks;
+    for (int i = part * 1024 + threadIdx.x; i < min(kv_heads * vd, (part + 1) * 1024); i += blockDim.x)
       v_cache[(((size_t)page * kv_heads + i / vd) * vd + i % vd) * page_size + slot] = v[i];
   }
 }
@@ -135,12 +139,15 @@ extern "C" int ns_unit_kv_write(void* qkv, int stride, const int* positions, con
                                 void* k_cache, void* v_cache, int n_tokens, int heads, int kv_heads, int hd, int vd, int page_size,
                                 float eps, int own_kv, int dtype, hipStream_t stream) {
   if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || hd <= 0 || vd <= 0 || page_size <= 0) return NS_ERR_BAD_ARG;
+  const int vec_blocks = (heads + (own_kv ? kv_heads : 0) + 3) / 4, copy_blocks = own_kv ? (kv_heads * vd + 1023) / 1024 : 0;
+  if (vec_blocks + copy_blocks > 65535) return NS_ERR_BAD_ARG;
+  const dim3 grid(n_tokens, vec_blocks + copy_blocks);
   if (dtype == NS_DTYPE_F32)
-    unit_kv_write_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)qkv, stride, positions, token_req, block_table, table_stride,
-                                                               (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, vd, page_size, eps, own_kv);
+    unit_kv_write_kernel<float><<<grid, 256, 0, stream>>>((float*)qkv, stride, positions, token_req, block_table, table_stride,
+                                                               (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, vd, page_size, eps, own_kv, vec_blocks);
   else if (dtype == NS_DTYPE_BF16)
-    unit_kv_write_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((bf16_t*)qkv, stride, positions, token_req, block_table, table_stride,
-                                                                (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, vd, page_size, eps, own_kv);
+    unit_kv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)qkv, stride, positions, token_req, block_table, table_stride,
+                                                                (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, vd, page_size, eps, own_kv, vec_blocks);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();

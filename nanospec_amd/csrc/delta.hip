@@ -85,37 +85,45 @@ extern "C" int ns_conv_silu_carry(float* out, const void* x, int x_stride, const
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ float softplus_f(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
+// grid (tokens, Y): the first ceil(2 G / 4) blocks of a token take one vector a wave; the others 1,024 decays each (and
+// the first of them the write strengths), so that no wave walks through a chain of dependent loads.
 template <typename T>
 __global__ void delta_prep_kernel(float* __restrict__ qkv, int C, float* __restrict__ g, float* __restrict__ beta, const T* __restrict__ a,
                                   int a_stride, const T* __restrict__ bp, int b_stride, const float* __restrict__ dt_bias,
-                                  const float* __restrict__ a_log, int H, int G, int D) {
-  const int r = blockIdx.x, lane = threadIdx.x & (NS_WAVE - 1), wave = threadIdx.x / NS_WAVE, nw = blockDim.x / NS_WAVE;
-  float* row = qkv + (size_t)r * C;
-  const float q_scale = 1.f / sqrtf((float)D);
-  for (int vec = wave; vec < 2 * G; vec += nw) {  // q heads, then k heads
-    float* p = row + (size_t)vec * D;
+                                  const float* __restrict__ a_log, int H, int G, int D, int norm_blocks) {
+  const int r = blockIdx.x, lane = threadIdx.x & (NS_WAVE - 1), wave = threadIdx.x / NS_WAVE;
+  if ((int)blockIdx.y < norm_blocks) {
+    const int vec = blockIdx.y * 4 + wave;  // q heads, then k heads
+    if (vec >= 2 * G) return;
+    float* p = qkv + (size_t)r * C + (size_t)vec * D;
     float ss = 0.f;
     for (int d = lane; d < D; d += NS_WAVE) ss = fmaf(p[d], p[d], ss);
     ss = wave_sum(ss);
-    const float f = (vec < G ? q_scale : 1.f) / sqrtf(ss + 1e-6f);
+    const float f = (vec < G ? 1.f / sqrtf((float)D) : 1.f) / sqrtf(ss + 1e-6f);
     for (int d = lane; d < D; d += NS_WAVE) p[d] *= f;
+    return;
   }
-  for (int i = threadIdx.x; i < H * D; i += blockDim.x) {
+  const int part = blockIdx.y - norm_blocks;
+  for (int i = part * 1024 + threadIdx.x; i < min(H * D, (part + 1) * 1024); i += blockDim.x) {
     const float z = to_f(a[(size_t)r * a_stride + i]) + dt_bias[i];
     g[(size_t)r * H * D + i] = expf(-expf(a_log[i / D]) * softplus_f(z));
   }
-  for (int h = threadIdx.x; h < H; h += blockDim.x) beta[(size_t)r * H + h] = 1.f / (1.f + expf(-to_f(bp[(size_t)r * b_stride + h])));
+  if (part == 0)
+    for (int h = threadIdx.x; h < H; h += blockDim.x) beta[(size_t)r * H + h] = 1.f / (1.f + expf(-to_f(bp[(size_t)r * b_stride + h])));
 }
 
 extern "C" int ns_delta_prep(float* qkv, int C, float* g, float* beta, const void* a, int a_stride, const void* bp, int b_stride,
                              const float* dt_bias, const float* a_log, int n_tokens, int H, int G, int D, int dtype, hipStream_t stream) {
   if (n_tokens <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || C < 2 * G * D) return NS_ERR_BAD_ARG;
+  const int norm_blocks = (2 * G + 3) / 4, decay_blocks = (H * D + 1023) / 1024;
+  if (norm_blocks + decay_blocks > 65535) return NS_ERR_BAD_ARG;
+  const dim3 grid(n_tokens, norm_blocks + decay_blocks);
   if (dtype == NS_DTYPE_F32)
-    delta_prep_kernel<float><<<n_tokens, 256, 0, stream>>>(qkv, C, g, beta, (const float*)a, a_stride, (const float*)bp, b_stride, dt_bias,
-                                                            a_log, H, G, D);
+    delta_prep_kernel<float><<<grid, 256, 0, stream>>>(qkv, C, g, beta, (const float*)a, a_stride, (const float*)bp, b_stride, dt_bias,
+                                                        a_log, H, G, D, norm_blocks);
   else if (dtype == NS_DTYPE_BF16)
-    delta_prep_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(qkv, C, g, beta, (const bf16_t*)a, a_stride, (const bf16_t*)bp, b_stride,
-                                                             dt_bias, a_log, H, G, D);
+    delta_prep_kernel<bf16_t><<<grid, 256, 0, stream>>>(qkv, C, g, beta, (const bf16_t*)a, a_stride, (const bf16_t*)bp, b_stride,
+                                                         dt_bias, a_log, H, G, D, norm_blocks);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();
