@@ -189,6 +189,9 @@ class ModelSpec:
     # the residual stream between the blocks: 0 = one stream in the model's precision; S >= 1 = S copies in 32-bit, all
     # equal to the embedding's output at the start and added up before the last norm (blocks of kind "streams")
     streams: int = 0
+    # tensor-name prefixes that a checkpoint may hold although the model reads nothing under them (the tensors of a
+    # sublayer that a layer does not have); anything else that is unexpected is an error
+    unread_prefixes: tuple[str, ...] = field(default_factory=tuple)
 
     def __post_init__(self) -> None:
         for pos, call in enumerate(self.run_order):

@@ -166,6 +166,8 @@ class VuzelixConfig:
             embed_scale=self.embedding_scale,
             logit_softcap=self.logit_softcap,
             streams=self.streams or 1,
+            # a layer without a feed-forward has no second sublayer: its norm, hyper-connection and matrices are not read
+            unread_prefixes=tuple(f"l{i}.{name}" for i, l in enumerate(self.layers) if l.ff is None for name in ("norm2", "hc2.", "mlp.")),
         )
 
 

@@ -14,6 +14,7 @@
 #include "common.h"
 
 #define AG_THREADS 256
+#define AG_MAX_VD 1024  // the largest value size (a thread holds up to four channels of the output)
 
 template <typename T>
 __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
@@ -35,7 +36,8 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
   int lo = window > 0 ? max(0, pos - window + 1) : 0;
   if (chunk > 0) lo = max(lo, pos / chunk * chunk);
   const float inv_cap = cap > 0.f ? 1.f / cap : 0.f;
-  float m = -INFINITY, l = 0.f, acc = 0.f;  // acc: channel `tid` of the output (tid < vd)
+  float m = -INFINITY, l = 0.f;
+  float acc[AG_MAX_VD / AG_THREADS] = {};  // channels tid, tid + 256, ... of the output
   for (int c0 = (lo / AG_THREADS) * AG_THREADS; c0 <= pos; c0 += AG_THREADS) {
     const int key = c0 + tid;
     const bool valid = key >= lo && key <= pos;
@@ -54,27 +56,34 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     const float alpha = m == -INFINITY ? 0.f : expf(m - m_new);
     l = l * alpha + csum;
     m = m_new;
-    if (tid < vd) {
-      acc *= alpha;
-      const int hi = min(AG_THREADS, pos - c0 + 1);
-      for (int j = max(0, lo - c0); j < hi; ++j) {
-        const int kj = c0 + j;
-        const int page = table[kj / page_size];
-        const T* vp = v_cache + (((size_t)page * kv_heads + kvh) * vd + tid) * page_size + kj % page_size;
-        acc = fmaf(p_s[j], to_f(*vp), acc);
+#pragma unroll
+    for (int ci = 0; ci < AG_MAX_VD / AG_THREADS; ++ci) {
+      const int ch = tid + ci * AG_THREADS;
+      if (ch < vd) {
+        float a = acc[ci] * alpha;
+        const int hi = min(AG_THREADS, pos - c0 + 1);
+        for (int j = max(0, lo - c0); j < hi; ++j) {
+          const int kj = c0 + j;
+          const int page = table[kj / page_size];
+          const T* vp = v_cache + (((size_t)page * kv_heads + kvh) * vd + ch) * page_size + kj % page_size;
+          a = fmaf(p_s[j], to_f(*vp), a);
+        }
+        acc[ci] = a;
       }
     }
     __syncthreads();
   }
   if (sink) l += expf(-m);  // the term of score 0, in the units of the running maximum
-  if (tid < vd) out[((size_t)t * heads + h) * vd + tid] = from_f<T>(acc / l);
+#pragma unroll
+  for (int ci = 0; ci < AG_MAX_VD / AG_THREADS; ++ci)
+    if (tid + ci * AG_THREADS < vd) out[((size_t)t * heads + h) * vd + tid + ci * AG_THREADS] = from_f<T>(acc[ci] / l);
 }
 
 extern "C" int ns_attn_generic(void* out, const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                const int* token_req, const int* positions, const int* block_table, int table_stride,
                                int n_tokens, int heads, int kv_heads, int hd, int vd, int page_size, float scale, int window,
                                int chunk, float cap, int sink, int dtype, hipStream_t stream) {
-  if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || hd <= 0 || hd > 1024 || vd <= 0 || vd > AG_THREADS || page_size <= 0 ||
+  if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || hd <= 0 || hd > 1024 || vd <= 0 || vd > AG_MAX_VD || page_size <= 0 ||
       window < 0 || chunk < 0 || cap < 0.f)
     return NS_ERR_BAD_ARG;
   if (heads > 65535) return NS_ERR_BAD_ARG;

@@ -663,14 +663,14 @@ def _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim, v_dim: int 
 def attention_generic(q, out, k_cache, v_cache, token_req, positions, block_table, heads: int, kv_heads: int, head_dim: int,
                       scale: float, window: int = 0, v_dim: int | None = None, chunk: int = 0, cap: float = 0.0,
                       sink: bool = False) -> torch.Tensor:
-    """Attention of every token's query over its request's pages; any key size up to 1024 and value size up to 256, either
+    """Attention of every token's query over its request's pages; any key and value size up to 1024, either
     dtype.  ``chunk`` > 0: a query sees no key before the start of its own chunk of positions; ``cap`` > 0: scores become
     cap * tanh(score / cap); ``sink``: one more term of score 0 without a value in the soft-max's denominator."""
     v_dim = head_dim if v_dim is None else v_dim
     page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim, v_dim)
     _i32(token_req, "token_req"), _i32(positions, "positions"), _i32(block_table, "block_table")
-    if head_dim > 1024 or v_dim > 256:
-        raise KernelRefused(f"attention_generic takes key sizes up to 1024 and value sizes up to 256, not {head_dim} and {v_dim}")
+    if head_dim > 1024 or v_dim > 1024:
+        raise KernelRefused(f"attention_generic takes key and value sizes up to 1024, not {head_dim} and {v_dim}")
     n = q.shape[0]
     _check(build.core().ns_attn_generic(_ptr(out), _ptr(q), c_int(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(token_req),
                                         _ptr(positions), _ptr(block_table), c_int(block_table.stride(0)), c_int(n), c_int(heads),

@@ -75,7 +75,7 @@ class DecoderModel:
         spec = self.spec
         full = self.wanted()
         wanted = {k: v[0] for k, v in full.items()}
-        wsource.check(source, wanted, optional={spec.head_name} if spec.tie_head else frozenset())
+        wsource.check(source, wanted, optional={spec.head_name} if spec.tie_head else frozenset(), unread_prefixes=spec.unread_prefixes)
         self.dtype, self.device = dtype, torch.device(device)
         if layouts != "auto" and layouts not in LAYOUTS:
             raise ValueError(f"layouts={layouts!r}: use 'auto', 'both' or 'tiled'")

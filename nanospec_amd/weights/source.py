@@ -81,13 +81,13 @@ class SafetensorsSource:
         return _normalise(self._of[name].get_tensor(name))
 
 
-def check(source, wanted: dict[str, tuple[int, ...]], optional: set[str] = frozenset()) -> None:
+def check(source, wanted: dict[str, tuple[int, ...]], optional: set[str] = frozenset(), unread_prefixes: tuple[str, ...] = ()) -> None:
     """Compare a source's header with the tensors a model wants; raise one WeightError that lists
     everything wrong.  ``optional`` names may be absent (a tied output head).  A wanted size of None fits any size (a part
-    that reads an inner size from the checkpoint itself)."""
+    that reads an inner size from the checkpoint itself).  Names under ``unread_prefixes`` may be present and are not read."""
     have = set(source.names())
     missing = sorted(n for n in wanted if n not in have and n not in optional)
-    unexpected = sorted(have - set(wanted))
+    unexpected = sorted(n for n in have - set(wanted) if not n.startswith(tuple(unread_prefixes)))
     fits = lambda have_shape, want: len(have_shape) == len(want) and all(w is None or w == h for h, w in zip(have_shape, want))
     wrong = [(n, source.shape(n), wanted[n]) for n in sorted(have & set(wanted)) if not fits(tuple(source.shape(n)), tuple(wanted[n]))]
     if missing or unexpected or wrong:

@@ -1,5 +1,5 @@
-"""Configurations at the edges of what the kernels take: head sizes in steps of 16 up to 256 (and one that is no multiple of
-16), widths and feed-forward sizes that are no multiple of 8 or of anything, vocabularies that are no power of two,
+"""Configurations at the edges of what the kernels take: head sizes in steps of 16 up to 256 (one that is no multiple of
+16, one of 272), widths and feed-forward sizes that are no multiple of 8 or of anything, vocabularies that are no power of two,
 one head, seven heads, ten query heads to a key/value head.  Every one must give the plain implementation's logits, in
 32-bit and in bfloat16, decoded token by token and in a mixed schedule, or be refused with a clear error: never a wrong
 result."""
@@ -42,6 +42,9 @@ CONFIGS = {
     # a head size that is no multiple of 16: the matrix-core attention does not take it, the plain kernel does
     "head24": cfg(vocab_size=90, hidden_size=96, intermediate_size=136, num_hidden_layers=1, num_attention_heads=4,
                   num_key_value_heads=2, head_dim=24),
+    # a head beyond the matrix-core kernels' 256: the plain kernel takes it (a thread holds two channels of the output)
+    "head272": cfg(vocab_size=50, hidden_size=64, intermediate_size=96, num_hidden_layers=1, num_attention_heads=1, num_key_value_heads=1,
+                   head_dim=272),
     "llama3_scaling_16x64": cfg(vocab_size=4099, hidden_size=1024, intermediate_size=2816, num_hidden_layers=2, num_attention_heads=16,
                                 num_key_value_heads=16, head_dim=64, rope_theta=500000.0,
                                 rope_scaling=dict(rope_type="llama3", factor=4.0, low_freq_factor=1.0, high_freq_factor=4.0,
@@ -90,15 +93,15 @@ def test_odd_sizes_match_plain(folders, name, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_a_head_size_beyond_the_kernels_is_refused(tmp_path, dtype):
-    """Heads of 272 channels: no attention kernel takes them.  The step raises with the reason; nothing is computed elsewhere."""
+    """Heads of 1,040 channels: no attention kernel takes them.  The step raises with the reason; nothing is computed elsewhere."""
     from nanospec_amd.config import LlamaConfig
     from nanospec_amd.engine.replay import Replayer
     from nanospec_amd.kernels.ops import KernelRefused
     from nanospec_amd.loader import load_model
     from nanospec_amd.weights import write_model_folder
 
-    c = cfg(vocab_size=50, hidden_size=64, intermediate_size=96, num_hidden_layers=1, num_attention_heads=1, num_key_value_heads=1, head_dim=272)
+    c = cfg(vocab_size=50, hidden_size=64, intermediate_size=96, num_hidden_layers=1, num_attention_heads=1, num_key_value_heads=1, head_dim=1040)
     folder = write_model_folder(tmp_path / "wide_head", LlamaConfig.from_hf(c), 1, torch.float32)
     rep = Replayer(load_model(folder, dtype=dtype), 64, page_size=16)
-    with pytest.raises(KernelRefused, match="256"):
+    with pytest.raises(KernelRefused, match="1024"):
         rep.step([{"id": "a", "tokens": [1, 2, 3], "want": [2]}], [])

@@ -101,6 +101,14 @@ def test_weights_with_an_inner_size_of_their_own_fit():
     check(Header({"a": (7, 48)}), {"a": (None, 48)})
     with pytest.raises(WeightError):
         check(Header({"a": (7, 40)}), {"a": (None, 48)})
+    # what a checkpoint holds for a sublayer that a layer does not have is not read; anything else unexpected is an error
+    from nanospec_amd.config import resolve
+
+    _, spec = resolve(CFG)
+    assert spec.unread_prefixes == ("l1.norm2", "l1.hc2.", "l1.mlp.")
+    check(Header({"a": (2,), "l1.norm2": (48,), "l1.hc2.in": (2,)}), {"a": (2,)}, unread_prefixes=spec.unread_prefixes)
+    with pytest.raises(WeightError):
+        check(Header({"a": (2,), "l0.extra": (48,)}), {"a": (2,)}, unread_prefixes=spec.unread_prefixes)
 
 
 # ------------------------------------------------------------------------------------------------ the plain implementation

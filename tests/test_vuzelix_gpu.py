@@ -242,6 +242,23 @@ def test_greedy_generation_through_the_engine(folders, name, dtype):
         assert len(ours) == new
 
 
+def test_preempted_requests_start_their_state_again(folders):
+    """A pool too small for all requests with the policy that releases the newest one and recomputes it later: its state
+    slot is zeroed again at its second admission, and the tokens are those of a pool that is large enough."""
+    from nanospec_amd import Engine, EngineConfig, SamplingParams
+
+    name, page = "P", CONFIGS["P"]["page"]
+    model = engine_model(folders[name], name, torch.float32)
+    prompts = [t[:20] for t in sequences(name).values() if len(t) >= 20] * 2
+    new = 30
+    calm = Engine(model, EngineConfig(num_blocks=128, block_size=page)).generate(prompts, SamplingParams(max_tokens=new))
+    eng = Engine(model, EngineConfig(num_blocks=23, block_size=page, on_exhaustion="preempt", prefill_chunk=16))
+    rough = eng.generate(prompts, SamplingParams(max_tokens=new))
+    assert eng.sched.preempted_total > 0, "the pool was meant to run out"
+    assert rough == calm
+    eng.cache.check()
+
+
 def test_the_command_line_generates(folders):
     import subprocess
     import sys
@@ -589,7 +606,7 @@ def step_context(lens, starts, tables, want=()):
     return StepContext(layout, torch.from_numpy(host).to(DEV), Arena(DEV), max_position=max_kv - 1, max_kv_len=max_kv, max_chunk_kv=chunk_kv)
 
 
-@pytest.mark.parametrize("hd,page", [(64, 16), (128, 16), (32, 16), (16, 8)])
+@pytest.mark.parametrize("hd,page", [(64, 16), (128, 16), (32, 16), (16, 8), (48, 16)])
 @pytest.mark.parametrize("G,group", [(2, 4), (3, 1)])
 def test_matrix_core_attention_with_options(hd, page, G, group):
     """The bfloat16 tile kernels with chunks, capped scores and the sink, as the attention part launches them: a long
