@@ -194,50 +194,67 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
   const float* v_src = qkv + (size_t)2 * p.G * D + (size_t)h * E + j0;
   const float* g_src = g + (size_t)h * D;
   const int stage_elems = p.stage_tokens * p.tok_stride;
-  // A thread fetches groups of four floats; every part of a token's record starts at a multiple of four.  The loads are
-  // issued without a branch around any of them (addresses of groups that hold nothing are bent to the start of the
-  // source and their values dropped), so that all of a stage's loads are in flight together.
-  // (what is kept of a loaded group is decided when it is parked, so that nothing here waits for a load)
-  struct Stage {
-    float4 v[ND_STAGE_REGS];
-    float bt[ND_STAGE_REGS];
-    unsigned keep, is_beta;  // four bits a group: which of its floats are kept; one bit a group: its first float is beta
-  };
-  auto fetch = [&](Stage& st, int first) {
+  // A thread fetches groups of four floats; every part of a token's record starts at a multiple of four.  Which group of
+  // which token's record a thread's i-th load is does not change from stage to stage, so source, row pitch and what is
+  // kept of it are worked out once; a stage's loads then differ only in the row, and are issued without a branch around
+  // any of them (a group that holds nothing reads the start of its source and is dropped when it is parked), so that
+  // all of a stage's loads are in flight together and nothing waits for one before the stage's tokens are done.
+  const float* src_of[ND_STAGE_REGS];
+  int pitch_of[ND_STAGE_REGS], token_of[ND_STAGE_REGS];
+  unsigned keep = 0, is_beta = 0;  // four bits a group: which of its floats are kept; one bit a group: its first float is beta
+  {
     int tt = threadIdx.x * 4 / p.tok_stride, off = threadIdx.x * 4 - tt * p.tok_stride;  // of element e, kept up as e grows by 1024
-    st.keep = st.is_beta = 0;
 #pragma unroll
     for (int i = 0; i < ND_STAGE_REGS; ++i) {
       const int e = (threadIdx.x + i * 256) * 4;
-      const int r = min(first + tt, r1 - 1);
-      const bool live = e < stage_elems && first + tt < r1;
+      const bool used = e < stage_elems;
       const int part = off < DL ? 0 : (off < 2 * DL ? 1 : (off < 3 * DL ? 2 : 3));
       const int within = off - part * DL, chunk = within / ND_PITCH, w = within - chunk * ND_PITCH;
       const int d = w < ND_ROWS ? chunk * ND_ROWS + w : 0x3fffffff;  // (the unused floats keep nothing)
       const int c = off - 3 * DL;
-      const float* src = part == 0 ? q_src + (size_t)r * p.C : (part == 1 ? k_src + (size_t)r * p.C : (part == 2 ? g_src + (size_t)r * p.H * D : v_src + (size_t)r * p.C));
       const int at = part < 3 ? d : c;
-      const int lim = !live ? 0 : (part < 3 ? D : min(COLS, E - j0));
-      if constexpr (VEC) {
-        st.v[i] = *reinterpret_cast<const float4*>(src + (at < lim ? at : 0));
-        st.keep |= (at < lim ? 0xfu : 0u) << (4 * i);
-      } else {
-        st.v[i] = float4{src[at < lim ? at : 0], src[at + 1 < lim ? at + 1 : 0], src[at + 2 < lim ? at + 2 : 0], src[at + 3 < lim ? at + 3 : 0]};
-        st.keep |= ((at < lim ? 1u : 0u) | (at + 1 < lim ? 2u : 0u) | (at + 2 < lim ? 4u : 0u) | (at + 3 < lim ? 8u : 0u)) << (4 * i);
-      }
-      st.bt[i] = beta[(size_t)r * p.H + h];
-      st.is_beta |= (live && part >= 3 && c == COLS ? 1u : 0u) << i;
+      const int lim = !used ? 0 : (part < 3 ? D : min(COLS, E - j0));
+      const float* src = part == 0 ? q_src : (part == 1 ? k_src : (part == 2 ? g_src : v_src));
+      const unsigned bits = VEC ? (at < lim ? 0xfu : 0u)
+                                : ((at < lim ? 1u : 0u) | (at + 1 < lim ? 2u : 0u) | (at + 2 < lim ? 4u : 0u) | (at + 3 < lim ? 8u : 0u));
+      src_of[i] = src + (bits ? at : 0);
+      pitch_of[i] = part == 2 ? p.H * D : p.C;
+      token_of[i] = tt;
+      keep |= bits << (4 * i);
+      is_beta |= (used && part >= 3 && c == COLS ? 1u : 0u) << i;
       off += 1024;
       while (off >= p.tok_stride) off -= p.tok_stride, ++tt;
+    }
+  }
+  struct Stage {
+    float4 v[ND_STAGE_REGS];
+    float bt[ND_STAGE_REGS];
+    unsigned live;  // one bit a group: its token is one of the request's
+  };
+  auto fetch = [&](Stage& st, int first) {
+    st.live = 0;
+#pragma unroll
+    for (int i = 0; i < ND_STAGE_REGS; ++i) {
+      const int r = min(first + token_of[i], r1 - 1);
+      st.live |= (first + token_of[i] < r1 ? 1u : 0u) << i;
+      const float* src = src_of[i] + (size_t)r * pitch_of[i];
+      if constexpr (VEC) {
+        st.v[i] = *reinterpret_cast<const float4*>(src);
+      } else {
+        const unsigned k = keep >> (4 * i);
+        st.v[i] = float4{src[0], src[k & 2u ? 1 : 0], src[k & 4u ? 2 : 0], src[k & 8u ? 3 : 0]};
+      }
+      st.bt[i] = beta[(size_t)r * p.H + h];
     }
   };
   auto park = [&](const Stage& st, float* buf) {
 #pragma unroll
     for (int i = 0; i < ND_STAGE_REGS; ++i) {
       const int e = (threadIdx.x + i * 256) * 4;
-      const unsigned k = st.keep >> (4 * i);
+      const bool live = (st.live >> i) & 1u;
+      const unsigned k = live ? keep >> (4 * i) : 0u;
       float4 val = {k & 1u ? st.v[i].x : 0.f, k & 2u ? st.v[i].y : 0.f, k & 4u ? st.v[i].z : 0.f, k & 8u ? st.v[i].w : 0.f};
-      if ((st.is_beta >> i) & 1u) val.x = st.bt[i];
+      if (live && ((is_beta >> i) & 1u)) val.x = st.bt[i];
       if (e < stage_elems) *reinterpret_cast<float4*>(buf + e) = val;
     }
   };
