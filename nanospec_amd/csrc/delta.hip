@@ -165,7 +165,7 @@ struct DeltaShape {
   int C, H, G, D, E, RG, Dl, cols, tok_stride, stage_tokens, vec4;
 };
 
-template <bool VEC, int RG>
+template <bool VEC, int RG, int ROWS>
 __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, const float* __restrict__ qkv,
                                                          const float* __restrict__ g, const float* __restrict__ beta,
                                                          float* __restrict__ state, size_t slot_stride, const int* __restrict__ qo_indptr,
@@ -175,19 +175,20 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
   const int r0 = qo_indptr[b], r1 = qo_indptr[b + 1];
   if (r1 <= r0) return;
   const int D = p.D, E = p.E;
-  constexpr int DL = RG * ND_PITCH, COLS = 256 / RG;
+  constexpr int PITCH = ROWS + 4;  // floats between two row groups' channels in LDS
+  constexpr int DL = RG * PITCH, COLS = 256 / RG;
   const int jl = threadIdx.x / RG, rg = threadIdx.x % RG;
   const int j0 = blockIdx.z * COLS, j = j0 + jl;
   const bool col_ok = j < E;
-  const int d0 = rg * ND_ROWS;
+  const int d0 = rg * ROWS;
   const int kh = h / (p.H / p.G);
   float* S = state + (size_t)state_slots[b] * slot_stride + (size_t)h * D * E;
-  float s[ND_ROWS];
+  float s[ROWS];
 #pragma unroll
-  for (int i = 0; i < ND_ROWS; ++i) s[i] = (col_ok && d0 + i < D) ? S[(size_t)(d0 + i) * E + j] : 0.f;
+  for (int i = 0; i < ROWS; ++i) s[i] = (col_ok && d0 + i < D) ? S[(size_t)(d0 + i) * E + j] : 0.f;
 
   // what element e of a stage that starts at row `first` is: token e / tok_stride, then q [Dl] | k [Dl] | g [Dl] | v [cols] | beta;
-  // in q, k and g the 16 channels of a row group are followed by four unused floats (ND_PITCH), so that the row groups'
+  // in q, k and g the 16 channels of a row group are followed by four unused floats (PITCH), so that the row groups'
   // 16-byte reads fall into different banks
   const float* q_src = qkv + (size_t)kh * D;
   const float* k_src = qkv + (size_t)p.G * D + (size_t)kh * D;
@@ -209,8 +210,8 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
       const int e = (threadIdx.x + i * 256) * 4;
       const bool used = e < stage_elems;
       const int part = off < DL ? 0 : (off < 2 * DL ? 1 : (off < 3 * DL ? 2 : 3));
-      const int within = off - part * DL, chunk = within / ND_PITCH, w = within - chunk * ND_PITCH;
-      const int d = w < ND_ROWS ? chunk * ND_ROWS + w : 0x3fffffff;  // (the unused floats keep nothing)
+      const int within = off - part * DL, chunk = within / PITCH, w = within - chunk * PITCH;
+      const int d = w < ROWS ? chunk * ROWS + w : 0x3fffffff;  // (the unused floats keep nothing)
       const int c = off - 3 * DL;
       const int at = part < 3 ? d : c;
       const int lim = !used ? 0 : (part < 3 ? D : min(COLS, E - j0));
@@ -276,23 +277,23 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
     // Two sets of operand registers take turns: the next token's operands are read from LDS into one while the chain of
     // the current token runs on the other (written out twice, so that no set is ever copied into the other).
     struct Operands {
-      float4 q[ND_ROWS / 4], k[ND_ROWS / 4], g[ND_ROWS / 4];
+      float4 q[ROWS / 4], k[ROWS / 4], g[ROWS / 4];
       float v, b;
     };
     auto read_token = [&](Operands& t, int tt) {
       const float* tok = buf + tt * p.tok_stride;
 #pragma unroll
-      for (int i = 0; i < ND_ROWS / 4; ++i) {
-        t.q[i] = reinterpret_cast<const float4*>(tok + rg * ND_PITCH)[i];
-        t.k[i] = reinterpret_cast<const float4*>(tok + DL + rg * ND_PITCH)[i];
-        t.g[i] = reinterpret_cast<const float4*>(tok + 2 * DL + rg * ND_PITCH)[i];
+      for (int i = 0; i < ROWS / 4; ++i) {
+        t.q[i] = reinterpret_cast<const float4*>(tok + rg * PITCH)[i];
+        t.k[i] = reinterpret_cast<const float4*>(tok + DL + rg * PITCH)[i];
+        t.g[i] = reinterpret_cast<const float4*>(tok + 2 * DL + rg * PITCH)[i];
       }
       t.v = tok[3 * DL + jl], t.b = tok[3 * DL + COLS];
     };
     auto chain = [&](const Operands& t) {
       float part[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < ND_ROWS / 4; ++i) {
+      for (int i = 0; i < ROWS / 4; ++i) {
         s[4 * i] *= t.g[i].x, s[4 * i + 1] *= t.g[i].y, s[4 * i + 2] *= t.g[i].z, s[4 * i + 3] *= t.g[i].w;
         part[0] = fmaf(t.k[i].x, s[4 * i], part[0]);
         part[1] = fmaf(t.k[i].y, s[4 * i + 1], part[1]);
@@ -303,7 +304,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
       const float u = t.b * (t.v - dot);
       float acc[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int i = 0; i < ND_ROWS / 4; ++i) {
+      for (int i = 0; i < ROWS / 4; ++i) {
         s[4 * i] = fmaf(t.k[i].x, u, s[4 * i]);
         s[4 * i + 1] = fmaf(t.k[i].y, u, s[4 * i + 1]);
         s[4 * i + 2] = fmaf(t.k[i].z, u, s[4 * i + 2]);
@@ -332,7 +333,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
     cur ^= 1;
   }
 #pragma unroll
-  for (int i = 0; i < ND_ROWS; ++i)
+  for (int i = 0; i < ROWS; ++i)
     if (col_ok && d0 + i < D) S[(size_t)(d0 + i) * E + j] = s[i];
 }
 
@@ -341,9 +342,12 @@ extern "C" int ns_delta_scan(float* o, const float* qkv, int C, const float* g, 
   if (n_reqs <= 0 || H <= 0 || G <= 0 || H % G || D <= 0 || D > ND_ROWS * NS_WAVE || E <= 0 || H > 65535) return NS_ERR_BAD_ARG;
   DeltaShape p;
   p.C = C, p.H = H, p.G = G, p.D = D, p.E = E;
+  // A thread owns 8 key channels of a column where the key size allows it (more, shorter chains: a token's step is
+  // latency, and a single request leaves most of the GPU idle anyway), 16 beyond 512 channels.
+  const int rows = D <= 8 * NS_WAVE ? 8 : ND_ROWS;
   p.RG = 1;
-  while (p.RG * ND_ROWS < D) p.RG *= 2;
-  p.Dl = p.RG * ND_PITCH;
+  while (p.RG * rows < D) p.RG *= 2;
+  p.Dl = p.RG * (rows + 4);
   p.cols = 256 / p.RG;
   p.tok_stride = 3 * p.Dl + ((p.cols + 1 + 3) / 4) * 4;
   p.stage_tokens = ND_STAGE_FLOATS / p.tok_stride;
@@ -354,10 +358,13 @@ extern "C" int ns_delta_scan(float* o, const float* qkv, int C, const float* g, 
   const int zb = (E + p.cols - 1) / p.cols;
   if (zb > 65535) return NS_ERR_BAD_ARG;
   const dim3 grid(n_reqs, H, zb);
-#define ND_LAUNCH(R)                                                                                                             \
-  case R:                                                                                                                         \
-    if (p.vec4) delta_scan_kernel<true, R><<<grid, 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p); \
-    else delta_scan_kernel<false, R><<<grid, 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p);       \
+#define ND_LAUNCH2(R, W)                                                                                                               \
+  if (p.vec4) delta_scan_kernel<true, R, W><<<grid, 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p); \
+  else delta_scan_kernel<false, R, W><<<grid, 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p)
+#define ND_LAUNCH(R)                    \
+  case R:                               \
+    if (rows == 8) { ND_LAUNCH2(R, 8); } \
+    else { ND_LAUNCH2(R, ND_ROWS); }    \
     break
   switch (p.RG) {
     ND_LAUNCH(1);
@@ -368,6 +375,7 @@ extern "C" int ns_delta_scan(float* o, const float* qkv, int C, const float* g, 
     ND_LAUNCH(32);
     default: ND_LAUNCH(64);
   }
+#undef ND_LAUNCH2
 #undef ND_LAUNCH
   return ns_launch_status();
 }
