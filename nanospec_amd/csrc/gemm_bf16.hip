@@ -25,6 +25,8 @@ typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
 #define EPI_ROPE_KV 2
 #define EPI_RESID_NORM 3
 #define EPI_GATED_HALF 4
+#define EPI_ACT 5  // an activation on the result, which is rounded to bfloat16 first as a separate kernel would find it: 0 the
+                   // tanh form of GELU, 1 SiLU (NormLink::act)
 // EPI_GATED_HALF is EPI_SILU_MUL with half the work per workgroup: the 16 rows of a workgroup's matrix instruction are 8
 // rows of the gate matrix and the same 8 rows of the up matrix (a lane is free to take its 16 bytes from any row of
 // either tiled matrix), placed so that a gate row's sum and its up row's sum come out in the same lane.  Twice as many
@@ -52,6 +54,7 @@ struct NormLink {
   bf16_t* x_next;       // [M, resid_stride]
   float* ssq_out;       // [M][workgroups]
   int resid_stride;
+  int act;              // EPI_ACT: which activation
 };
 
 __device__ __forceinline__ bf16x8 load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
@@ -277,6 +280,10 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
       if (nl.ssq_in) u *= rinv_s[m];
       s = s / (1.f + expf(-s)) * u;
     }
+    if (EPI == EPI_ACT) {
+      const float z = (float)(bf16_t)s;
+      s = nl.act == 0 ? 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z))) : z / (1.f + expf(-z));
+    }
     out[(size_t)m * out_stride + n] = (OutT)s;
   }
 }
@@ -300,6 +307,9 @@ static int launch_tiled(void* out, const void* x, const void* w, const void* w2,
   } else if (epi == EPI_ROPE_KV) {
     if (out_f32 || MT != 1) return NS_ERR_UNSUPPORTED;
     gemm_tiled_kernel<1, WAVES, EPI_ROPE_KV, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride, rk, nl);
+  } else if (epi == EPI_ACT) {
+    if (out_f32) return NS_ERR_UNSUPPORTED;
+    gemm_tiled_kernel<MT, WAVES, EPI_ACT, bf16_t><<<grid, WAVES * 64, 0, stream>>>((bf16_t*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride, rk, nl);
   } else if (out_f32) {
     gemm_tiled_kernel<MT, WAVES, EPI_STORE, float><<<grid, WAVES * 64, 0, stream>>>((float*)out, xb, wb, nullptr, M, N, K, x_stride, out_stride, rk, nl);
   } else {
@@ -334,10 +344,12 @@ static int tiled_dispatch(void* out, const void* x, const void* wt, const void* 
 // ssq_in (may be null): x holds rows that a norm's weight has scaled but its 1/rms has not; see NormLink.
 extern "C" int ns_gemm_tiled_bf16(void* out, const void* x, const void* wt, const void* wt2, int M, int N, int K,
                                   int x_stride, int out_stride, int epi, int out_f32, int waves, const float* ssq_in,
-                                  int parts_in, int norm_dim, float eps, hipStream_t stream) {
-  if (epi != EPI_STORE && epi != EPI_SILU_MUL && epi != EPI_GATED_HALF) return NS_ERR_BAD_ARG;
+                                  int parts_in, int norm_dim, float eps, int act, hipStream_t stream) {
+  if (epi != EPI_STORE && epi != EPI_SILU_MUL && epi != EPI_GATED_HALF && epi != EPI_ACT) return NS_ERR_BAD_ARG;
+  if (epi == EPI_ACT && (act < 0 || act > 1)) return NS_ERR_BAD_ARG;
   RopeKvParams rk = {};
   NormLink nl = {};
+  nl.act = act;
   nl.ssq_in = ssq_in; nl.parts_in = parts_in; nl.inv_dim = norm_dim > 0 ? 1.f / (float)norm_dim : 0.f; nl.eps = eps;
   return tiled_dispatch(out, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, waves, rk, nl, stream);
 }

@@ -357,10 +357,14 @@ GATED_HALF_ROWS = 4  # up to this many rows the gated product runs half a row ti
 
 
 def linear_tiled(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
-                 out_f32: bool = False, waves: int = 0, halves: bool | None = None) -> torch.Tensor:
+                 out_f32: bool = False, waves: int = 0, halves: bool | None = None, act: str | None = None) -> torch.Tensor:
     """bfloat16 x @ w.T for at most 64 rows from a tiled weight; with ``w2``: silu(x @ w.T) * (x @ w2.T).  ``x`` may be a
     ``PreNormed`` (at most 16 rows).  ``halves`` (with ``w2``, at most 16 rows): a workgroup takes 8 rows of each matrix
-    instead of 16, which spreads a number of row tiles that is no multiple of the compute units evenly; None: by rows."""
+    instead of 16, which spreads a number of row tiles that is no multiple of the compute units evenly; None: by rows.
+    ``act`` (one of ``ACTIVATIONS``, not with ``w2`` or 32-bit results): the activation of the result, which is rounded to
+    bfloat16 first, so that the values are those of ``activation`` after this product."""
+    if act is not None and (w2 is not None or out_f32 or act not in ACTIVATIONS):
+        raise KernelRefused("linear_tiled: an activation goes with one matrix, a bfloat16 result and a known name")
     pre = x if isinstance(x, PreNormed) else None
     if pre is not None:
         x = pre.x
@@ -380,11 +384,12 @@ def linear_tiled(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight 
         waves = 8 if w.k >= 8192 or ((w.n // 16 < 512 or m > 8) and w.k >= 2048) else 4
     if halves is None:  # (with 3 or 4 rows only where whole row tiles would not spread evenly over 256 compute units)
         halves = m <= 2 or (m <= GATED_HALF_ROWS and -(-w.n // 16) % 256 != 0)
-    epi = 0 if w2 is None else (4 if halves and m <= 16 and not out_f32 else 1)
+    epi = (5 if act is not None else 0) if w2 is None else (4 if halves and m <= 16 and not out_f32 else 1)
     _check(build.core().ns_gemm_tiled_bf16(_ptr(out), _ptr(x), _ptr(w.data), _ptr(w2.data if w2 is not None else None), c_int(m),
                                            c_int(w.n), c_int(w.k), c_int(x.stride(0)), c_int(out.stride(0)),
                                            c_int(epi), c_int(1 if out_f32 else 0), c_int(waves),
-                                           *_prenorm_args(pre, m, "linear_tiled"), _stream()),
+                                           *_prenorm_args(pre, m, "linear_tiled"), c_int(ACTIVATIONS[act] if act is not None else 0),
+                                           _stream()),
            "linear_tiled")
     return out
 

@@ -33,8 +33,8 @@ class DenseFF:
 
     def forward(self, ctx, x, out: torch.Tensor | None = None):
         n = x.shape[0]
-        mid = self.up(x, out=ctx.arena.take((n, self.spec.intermediate), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)
-        ops.activation(mid, self.spec.activation)
+        mid = self.up(x, out=ctx.arena.take((n, self.spec.intermediate), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured,
+                      act=self.spec.activation)
         return self.down(mid, out=out if out is not None else ctx.arena.take((n, self.spec.hidden), x.dtype), arena=ctx.arena,
                          plain_copy=not ctx.captured)
 

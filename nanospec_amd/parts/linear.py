@@ -148,10 +148,18 @@ class LinearWeight:
         out = link.x_next if link.x_next is not None else take((m, self.n), x.dtype)
         return self(x, out=out, arena=arena, plain_copy=plain_copy)
 
-    def __call__(self, x, out: torch.Tensor | None = None, out_f32: bool = False, arena=None, plain_copy: bool = False) -> torch.Tensor:
+    def __call__(self, x, out: torch.Tensor | None = None, out_f32: bool = False, arena=None, plain_copy: bool = False,
+                 act: str | None = None) -> torch.Tensor:
         """``arena``: where the workspace of the 17-to-64-row kernel comes from (``ctx.arena``); without it it is allocated.
         ``x`` may be a ``PreNormed`` where ``links_norms`` holds.  ``plain_copy``: where only the re-laid copy is kept, many
-        rows may go to the library through a plain copy of the matrix in scratch (see ``UNTILE_MIN_ROWS``)."""
+        rows may go to the library through a plain copy of the matrix in scratch (see ``UNTILE_MIN_ROWS``).  ``act``: an
+        activation (``ops.ACTIVATIONS``) on the result: in the streaming kernel's epilogue for few rows, a kernel of its own
+        otherwise; the values are the same either way."""
+        if act is not None:
+            if (not out_f32 and self.tiled is not None and not isinstance(x, ops.PreNormed) and x.shape[0] <= STREAM_ROWS
+                    and x.dtype == self.dtype and ops.tiled_takes(x[:1], self.k)):
+                return ops.linear_tiled(x, self.tiled, out=out, act=act)
+            return ops.activation(self(x, out=out, out_f32=out_f32, arena=arena, plain_copy=plain_copy), act)
         if isinstance(x, ops.PreNormed):
             if not self.links_norms(x.shape[0]):
                 raise ops.KernelRefused("this product cannot take a pre-normed input (rows, layout or precision)")

@@ -343,6 +343,31 @@ def test_stream_write_and_read_in_one_pass(S, W, dtype):
     torch.testing.assert_close(h.cpu().double(), ref, **tol)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_dense_feed_forward_part(dtype):
+    """down(gelu(up x)) for few rows (the activation in the product's epilogue), some and many; the same values whichever
+    way the activation is applied."""
+    from nanospec_amd.config.spec import DenseFFSpec
+    from nanospec_amd.parts import build
+
+    torch.manual_seed(6)
+    part = build("ffn", DenseFFSpec(hidden=72, intermediate=200), "l.mlp.")
+    ws = {"l.mlp.up": torch.randn(200, 72) * 0.3, "l.mlp.down": torch.randn(72, 200) * 0.1}
+    assert {k: v[0] for k, v in part.wanted().items()} == {k: tuple(v.shape) for k, v in ws.items()}
+    part.load(ws.__getitem__, dtype, DEV)
+    x = torch.randn(200, 72).to(dtype)
+    outs = {}
+    for rows in (3, 40, 200):
+        ctx = step_context([rows], [0], [[0] * 16])
+        outs[rows] = part.forward(ctx, x[:rows].to(DEV)).cpu()
+        ref = pv.dense_ff(x[:rows].double(), {k: v.to(dtype).double() for k, v in ws.items()}, "l.mlp.")
+        tol = dict(rtol=1e-4, atol=1e-5) if dtype == torch.float32 else dict(rtol=3e-2, atol=3e-2)
+        torch.testing.assert_close(outs[rows].double(), ref, **tol)
+    # (the products of few, some and many rows add in different orders)
+    for rows in (40, 200):
+        assert (outs[3].float() - outs[rows][:3].float()).abs().max() <= (1e-5 if dtype == torch.float32 else 2e-2)
+
+
 def test_activation_is_the_tanh_form():
     from nanospec_amd.kernels import ops
 
