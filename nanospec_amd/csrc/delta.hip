@@ -36,6 +36,46 @@ __global__ void conv_silu_kernel(float* __restrict__ out, const T* __restrict__ 
   out[(size_t)r * C + c] = y / (1.f + expf(-y));
 }
 
+// The same for four neighbouring channels a thread, with 16-byte accesses to taps, carried inputs and results, for the
+// usual numbers of taps (so that the taps are registers) and channels that are a multiple of four.
+template <typename T, int K>
+__global__ void conv_silu_vec_kernel(float* __restrict__ out, const T* __restrict__ x, int x_stride, const float* __restrict__ taps,
+                                     const float* __restrict__ state, size_t slot_stride, size_t conv_off, const int* __restrict__ token_req,
+                                     const int* __restrict__ qo_indptr, const int* __restrict__ state_slots, int C) {
+  typedef T vec_t __attribute__((ext_vector_type(4)));
+  const int r = blockIdx.x, c = (blockIdx.y * blockDim.x + threadIdx.x) * 4;
+  if (c >= C) return;
+  const int b = token_req[r];
+  const int i = r - qo_indptr[b];
+  const float* carried = state + (size_t)state_slots[b] * slot_stride + conv_off;
+  float tp[4 * K];  // taps of channel c + e / K, tap e % K
+#pragma unroll
+  for (int e = 0; e < K; ++e) {
+    const float4 t = reinterpret_cast<const float4*>(taps + (size_t)c * K)[e];
+    tp[4 * e] = t.x, tp[4 * e + 1] = t.y, tp[4 * e + 2] = t.z, tp[4 * e + 3] = t.w;
+  }
+  float y[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < K; ++j) {
+    const int t = i - (K - 1) + j;
+    float v[4];
+    if (t >= 0) {
+      const vec_t xv = *reinterpret_cast<const vec_t*>(x + (size_t)(r - (K - 1) + j) * x_stride + c);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) v[e] = to_f(xv[e]);
+    } else {
+      const float4 cv = *reinterpret_cast<const float4*>(carried + (size_t)(K - 1 + t) * C + c);
+      v[0] = cv.x, v[1] = cv.y, v[2] = cv.z, v[3] = cv.w;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) y[e] = fmaf(tp[e * K + j], v[e], y[e]);
+  }
+  float4 res;
+  res.x = y[0] / (1.f + expf(-y[0])), res.y = y[1] / (1.f + expf(-y[1]));
+  res.z = y[2] / (1.f + expf(-y[2])), res.w = y[3] / (1.f + expf(-y[3]));
+  *reinterpret_cast<float4*>(out + (size_t)r * C + c) = res;
+}
+
 // After the convolution has read them: the carried inputs become the last K-1 inputs including this step's.
 template <typename T>
 __global__ void conv_carry_kernel(const T* __restrict__ x, int x_stride, float* __restrict__ state, size_t slot_stride, size_t conv_off,
@@ -60,7 +100,27 @@ extern "C" int ns_conv_silu_carry(float* out, const void* x, int x_stride, const
   if (dtype != NS_DTYPE_F32 && dtype != NS_DTYPE_BF16) return NS_ERR_UNSUPPORTED;
   const int bx = (C + 255) / 256;
   if (bx > 65535) return NS_ERR_BAD_ARG;
-  {
+  const size_t esize = dtype == NS_DTYPE_F32 ? 4 : 2;
+  const bool vec = C % 4 == 0 && x_stride % 4 == 0 && ((uintptr_t)x % (4 * esize)) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)taps % 16) == 0 &&
+                   ((uintptr_t)state % 16) == 0 && slot_stride % 4 == 0 && conv_off % 4 == 0 && K >= 2 && K <= 4;
+  if (vec) {
+    dim3 grid(n_tokens, (C / 4 + 255) / 256);
+#define ND_CONV(KK)                                                                                                                         \
+  case KK:                                                                                                                                  \
+    if (dtype == NS_DTYPE_F32)                                                                                                              \
+      conv_silu_vec_kernel<float, KK><<<grid, 256, 0, stream>>>(out, (const float*)x, x_stride, taps, state, slot_stride, conv_off, token_req, \
+                                                                qo_indptr, state_slots, C);                                                \
+    else                                                                                                                                    \
+      conv_silu_vec_kernel<bf16_t, KK><<<grid, 256, 0, stream>>>(out, (const bf16_t*)x, x_stride, taps, state, slot_stride, conv_off, token_req, \
+                                                                 qo_indptr, state_slots, C);                                               \
+    break
+    switch (K) {
+      ND_CONV(2);
+      ND_CONV(3);
+      default: ND_CONV(4);
+    }
+#undef ND_CONV
+  } else {
     dim3 grid(n_tokens, bx);
     if (dtype == NS_DTYPE_F32)
       conv_silu_kernel<float><<<grid, 256, 0, stream>>>(out, (const float*)x, x_stride, taps, state, slot_stride, conv_off, token_req,
@@ -130,7 +190,7 @@ extern "C" int ns_delta_prep(float* qkv, int C, float* g, float* beta, const voi
 }
 
 // ------------------------------------------------------------------------------------------------
-// The recurrence.  grid (requests, heads, blocks of columns); a thread = (column jl of the block, row group rg), lane
+// The recurrence.  grid (blocks of columns, heads, requests); a thread = (column jl of the block, row group rg), lane
 // = jl * RG + rg, RG a power of two (at most 64) with 16 RG >= D.  Channels beyond D carry zeros.
 //
 // A token's step is a chain (decay, dot product, lane exchange, update, dot product, lane exchange) that cannot start
@@ -171,14 +231,16 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(float* __restrict__ o, 
                                                          float* __restrict__ state, size_t slot_stride, const int* __restrict__ qo_indptr,
                                                          const int* __restrict__ state_slots, DeltaShape p) {
   __shared__ __attribute__((aligned(16))) float stage[2][ND_STAGE_FLOATS];
-  const int b = blockIdx.x, h = blockIdx.y;
+  // (the request is the slowest index of the launch: workgroups are dealt to the eight XCDs in turn, and with the request
+  // as the fastest index all workgroups of the one long request among eight would land on one XCD)
+  const int b = blockIdx.z, h = blockIdx.y;
   const int r0 = qo_indptr[b], r1 = qo_indptr[b + 1];
   if (r1 <= r0) return;
   const int D = p.D, E = p.E;
   constexpr int PITCH = ROWS + 4;  // floats between two row groups' channels in LDS
   constexpr int DL = RG * PITCH, COLS = 256 / RG;
   const int jl = threadIdx.x / RG, rg = threadIdx.x % RG;
-  const int j0 = blockIdx.z * COLS, j = j0 + jl;
+  const int j0 = blockIdx.x * COLS, j = j0 + jl;
   const bool col_ok = j < E;
   const int d0 = rg * ROWS;
   const int kh = h / (p.H / p.G);
@@ -356,8 +418,8 @@ extern "C" int ns_delta_scan(float* o, const float* qkv, int C, const float* g, 
   // 16-byte loads where every group of four that a thread fetches starts at a multiple of four floats
   p.vec4 = (D % 4 == 0 && E % 4 == 0 && C % 4 == 0 && ((uintptr_t)qkv % 16) == 0 && ((uintptr_t)g % 16) == 0) ? 1 : 0;
   const int zb = (E + p.cols - 1) / p.cols;
-  if (zb > 65535) return NS_ERR_BAD_ARG;
-  const dim3 grid(n_reqs, H, zb);
+  if (n_reqs > 65535) return NS_ERR_BAD_ARG;
+  const dim3 grid(zb, H, n_reqs);
 #define ND_LAUNCH2(R, W)                                                                                                               \
   if (p.vec4) delta_scan_kernel<true, R, W><<<grid, 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p); \
   else delta_scan_kernel<false, R, W><<<grid, 256, 0, stream>>>(o, qkv, g, beta, state, slot_stride, qo_indptr, state_slots, p)

@@ -384,24 +384,24 @@ def batch(lens, slots):
     return req, indptr, torch.tensor(slots, dtype=torch.int32, device=DEV)
 
 
-@pytest.mark.parametrize("K", [1, 2, 4, 7])
-def test_convolution_carries_its_inputs_across_steps(K):
+@pytest.mark.parametrize("C,pad,off", [(37, 5, 50), (40, 4, 52)], ids=["one_channel_a_thread", "four_channels_a_thread"])
+@pytest.mark.parametrize("K", [1, 2, 3, 4, 7])
+def test_convolution_carries_its_inputs_across_steps(K, C, pad, off):
     """Two requests in slots that are not in order, cut into steps shorter and longer than the taps; the other slots and
     what lies before the carried inputs stay as they were."""
     from nanospec_amd.kernels import ops
 
     torch.manual_seed(K)
-    C, pad = 37, 5
     taps = torch.randn(C, K)
     xs = {0: torch.randn(19, C + pad), 1: torch.randn(11, C + pad)}
-    state = torch.zeros(4, 50 + (K - 1) * C, device=DEV)
-    state[:, :50] = 7.0  # what lies before the carried inputs is not touched
+    state = torch.zeros(4, off + (K - 1) * C, device=DEV)
+    state[:, :off] = 7.0  # what lies before the carried inputs is not touched
     done = {0: 0, 1: 0}
     outs = {0: [], 1: []}
     for lens in ([1, 3], [2, 1], [1, 1], [6, 2], [9, 4]):
         x = torch.cat([xs[b][done[b] : done[b] + n] for b, n in enumerate(lens)])
         req, indptr, slots = batch(lens, [3, 1])
-        out = ops.conv_silu_carry(x.to(DEV), taps.to(DEV), state, 50, req, indptr, slots, out=torch.empty(sum(lens), C, device=DEV))
+        out = ops.conv_silu_carry(x.to(DEV), taps.to(DEV), state, off, req, indptr, slots, out=torch.empty(sum(lens), C, device=DEV))
         at = 0
         for b, n in enumerate(lens):
             outs[b].append(out[at : at + n].cpu())
@@ -409,7 +409,7 @@ def test_convolution_carries_its_inputs_across_steps(K):
             done[b] += n
     for b in (0, 1):
         torch.testing.assert_close(torch.cat(outs[b]).double(), pv.causal_conv_silu(xs[b][:, :C].double(), taps.double()), rtol=1e-5, atol=1e-5)
-    assert (state[:, :50] == 7.0).all() and (state[0] == torch.cat([torch.full((50,), 7.0), torch.zeros((K - 1) * C)]).to(DEV)).all()
+    assert (state[:, :off] == 7.0).all() and (state[0] == torch.cat([torch.full((off,), 7.0), torch.zeros((K - 1) * C)]).to(DEV)).all()
 
 
 @pytest.mark.parametrize("H,G,D,E", [(4, 2, 24, 40), (2, 2, 64, 20), (1, 1, 128, 128), (6, 3, 8, 72), (3, 1, 144, 16)])
