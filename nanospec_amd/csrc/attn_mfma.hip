@@ -521,7 +521,8 @@ constexpr int CPR = PS / 8 < 4 ? PS / 8 : 4;  // 16-byte pieces of a block that 
 // workgroups share a compute unit and each has a barrier of its own, so the two waves of a SIMD are not kept in the same
 // phase and one's matrix instructions run under the other's soft-max arithmetic.  It pays where the ranges are joined by
 // the second kernel anyway or the keys are many (the join costs a pass over the unnormalised sums).
-template <int SETS>
+// OPT: the options of AttnParams (chunks, capped scores, a sink) are honoured.
+template <int SETS, bool OPT = false>
 __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2))) void attn_prefill_kernel(AttnParams a) {
   if constexpr (SHARED_OK) {
     constexpr int K_BYTES = 32 * KROW * 2, V_BYTES = HD * VROW * 2, SET_BYTES = 2 * (K_BYTES + V_BYTES);
@@ -562,13 +563,22 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
       col_ok[u] = ti < n && head_ok;
       pos[u] = col_ok[u] ? kv_len - n + ti : -1;
       lo[u] = (col_ok[u] && a.window > 0) ? max(0, pos[u] - a.window + 1) : 0;
+      if constexpr (OPT) {
+        if (col_ok[u] && a.chunk > 0) lo[u] = max(lo[u], pos[u] / a.chunk * a.chunk);
+      }
     }
     // what the tile's tokens see, from the descriptor alone: the same in every wave
     const int first_pos = kv_len - n + t0, last_pos = kv_len - n + min(t0 + 31, n - 1);
     const int whi = last_pos + 1;                                                   // keys [wlo, whi) are seen by some token
-    const int wlo = a.window > 0 ? max(0, first_pos - a.window + 1) : 0;
+    int wlo = a.window > 0 ? max(0, first_pos - a.window + 1) : 0;
     const int full_hi = first_pos;                                                  // keys <= full_hi are seen by every token
-    const int full_lo = a.window > 0 ? max(0, last_pos - a.window + 1) : 0;         // ... if they are >= full_lo
+    int full_lo = a.window > 0 ? max(0, last_pos - a.window + 1) : 0;               // ... if they are >= full_lo
+    if constexpr (OPT) {
+      if (a.chunk > 0) {  // a token's chunk starts at a multiple of the chunk's size; the tile's tokens may lie in two chunks
+        wlo = max(wlo, first_pos / a.chunk * a.chunk);
+        full_lo = max(full_lo, last_pos / a.chunk * a.chunk);
+      }
+    }
     int tile_kb0 = wlo / 32, tile_kb1 = (whi + 31) / 32;
     if (a.splits > 1) {  // this workgroup's range of the tile's blocks; it may be empty
       const int per = (tile_kb1 - tile_kb0 + a.splits - 1) / a.splits;
@@ -699,6 +709,12 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
           f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
           for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][i], qw[u][i], acc, 0, 0, 0);
+          if constexpr (OPT) {
+            if (a.cap > 0.f) {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) acc[j] = capped(acc[j], a.cap_pre, a.cap);
+            }
+          }
           s[u][t] = acc;
         }
       // s[u][t][j] is key key_base + 8 g + 4 t + j of column c
@@ -840,6 +856,14 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
         for (int i = 0; i < NQ; ++i)
 #pragma unroll
           for (int t = 0; t < 2; ++t) s[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][i], qw[u][i], s[u][t], 0, 0, 0);
+        if constexpr (OPT) {
+          if (a.cap > 0.f) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t)
+#pragma unroll
+              for (int j = 0; j < 4; ++j) s[u][t][j] = capped(s[u][t][j], a.cap_pre, a.cap);
+          }
+        }
       };
       bf16x8 pf[2];
       float alpha[2];
@@ -907,7 +931,9 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
     // The first blocks of this set's range that every token of the tile sees wholly (an even number of them: rounds go in
     // pairs, one per register set) run the form without masks.  Both sets pass a barrier in every round, whichever form
     // a round takes.
-    const int seen_whole = a.window > 0 ? 0 : min(max((full_hi + 1) / 32 - kb0, 0), max(kb1 - kb0, 0)) & ~1;
+    // (with chunks: only if this set's first block already lies in the chunk of the tile's last token)
+    const bool bounded_below = a.window > 0 || (OPT && a.chunk > 0 && kb0 * 32 < full_lo);
+    const int seen_whole = bounded_below ? 0 : min(max((full_hi + 1) / 32 - kb0, 0), max(kb1 - kb0, 0)) & ~1;
     const bool all_heads = (y % hblks) * 4 + 3 < G;
     const int n_steady = (EVEN && all_heads) ? max(min(seen_whole, kb1 - kb0 - 4), 0) & ~1 : 0;
     int it = 0;
@@ -968,6 +994,9 @@ __global__ __launch_bounds__(SETS * 256) __attribute__((amdgpu_waves_per_eu(2)))
       // o[u][dt][j] is channel 16 dt + 4 g + j of column c
       if (a.splits == 1) {
         const size_t col = (size_t)(q0 + t0 + u * 16 + c) * a.heads + head;
+        if constexpr (OPT) {
+          if (a.sink) lsum[u] += fast_exp2(-m[u] * a.scale_log2);  // the term of score 0, in the units of the column's maximum
+        }
         const float inv = 1.f / lsum[u];
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt) {
@@ -1102,7 +1131,14 @@ extern "C" int ns_attn_mfma(void* out, void* part_o, void* part_ml, const void* 
   const long blocks = coop ? items : (items + 3) / 4;
   if (blocks > 0x7fffffffL) return NS_ERR_BAD_ARG;
   if (opt) {
-    if (qt == 2)
+    if (qt == 2 && SHARED_OK) {  // prompt portions: the 16x16 kernel that shares keys through LDS
+      const long wgs = (long)n_tiles * splits * kv_heads * ((G + 3) / 4);
+      if (wgs > 0x7fffffffL) return NS_ERR_BAD_ARG;
+      if (coop)
+        attn_prefill_kernel<1, true><<<(unsigned)wgs, 256, 0, stream>>>(a);
+      else
+        attn_prefill_kernel<2, true><<<(unsigned)wgs, 512, 0, stream>>>(a);
+    } else if (qt == 2)
       attn_mfma_kernel<2, false, false, true><<<(unsigned)blocks, 256, 0, stream>>>(a);
     else if (coop)
       attn_mfma_kernel<1, true, true, true><<<(unsigned)blocks, 256, 0, stream>>>(a);
