@@ -674,3 +674,64 @@ def test_matrix_core_attention_with_options(hd, page, G, group):
             torch.testing.assert_close(out[at : at + n].cpu().double().view(n, H, hd), ref, rtol=2e-2, atol=2e-2,
                                        msg=lambda m: f"request {b}, scale {scale}, cap {cap}, chunk {chunk}, sink {sink}: {m}")
             at += n
+
+
+def drawn_config(seed: int) -> tuple[dict, tuple[int, int]]:
+    """A small configuration drawn from everything the design lets a model choose: sizes, head counts, the order of the
+    layers, chunks, caps, scales, taps, streams, who borrows whose keys, which layers have no feed-forward."""
+    import random
+
+    rnd = random.Random(seed)
+    layers, owners = [], []
+    for i in range(rnd.randint(2, 6)):
+        ff = None if rnd.random() < 0.25 else rnd.choice((32, 56, 100, 200))
+        if rnd.random() < 0.4:
+            heads = rnd.choice((1, 2, 3, 4))
+            kvh = rnd.choice([k for k in (1, 2, 3, 4) if heads % k == 0])
+            layers.append(delta_layer(heads, kvh, rnd.choice((8, 16, 24, 32, 48)), rnd.choice((8, 16, 32, 40)), rnd.randint(1, 5), ff))
+            continue
+        mine = [o for o in owners if rnd.random() < 0.4]
+        if mine:
+            src = rnd.choice(mine)
+            kvh, dim, vdim = (layers[src]["mixer"][k] for k in ("kv_heads", "dim", "vdim"))
+        else:
+            src = None
+            kvh, dim = rnd.choice((1, 2, 3)), rnd.choice((8, 16, 24, 32, 64))
+            vdim = rnd.choice((dim, dim, 8, 16, 40, 64))
+            owners.append(i)
+        layers.append(attn_layer(kvh * rnd.choice((1, 2, 4)), kvh, dim, vdim, round(rnd.uniform(0.1, 0.6), 3), ff,
+                                 softcap=rnd.choice((None, 5.0, 20.0, 50.0)), chunk=rnd.choice((None, 5, 16, 33, 64)), kv_from=src))
+    cfg = {"architecture": "Vuzelix", "vocab": rnd.randint(50, 300), "width": rnd.choice((48, 64, 80, 136)), "layers": layers,
+           "norm": {"eps": rnd.choice((1e-5, 1e-6))}}
+    if rnd.random() < 0.7:
+        cfg["streams"] = rnd.randint(1, 5)
+    if rnd.random() < 0.7:
+        cfg["residual_mult"] = rnd.choice((0.3, 0.7, 1.5))
+    if rnd.random() < 0.6:
+        cfg["embedding"] = {"scale": rnd.choice((0.5, 2.0, 4.0))}
+    if rnd.random() < 0.6:
+        cfg["logit_softcap"] = rnd.choice((8.0, 30.0))
+    return cfg, (rnd.randint(4, 20), rnd.randint(4, 20))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("seed", range(8))
+def test_drawn_configurations_match_plain(tmp_path, seed, dtype):
+    """Eight configurations drawn at random: a prompt whole, with its last tokens decoded one by one, in portions, and
+    beside a second request."""
+    from dataclasses import replace
+
+    from nanospec_amd.config import VuzelixConfig
+    from nanospec_amd.loader import load_model
+    from nanospec_amd.weights import write_model_folder
+
+    cfg, ranks = drawn_config(seed)
+    folder = write_model_folder(tmp_path / "m", replace(VuzelixConfig.from_hf(cfg), decay_rank=ranks[0], gate_rank=ranks[1]), seed, torch.float32)
+    cfg_read, w = read_folder(folder, dtype)
+    seqs = {"a": random_tokens(70, cfg["vocab"], seed), "b": random_tokens(9, cfg["vocab"], seed + 100)}
+    ref = {rid: pv.forward(cfg_read, w, toks, torch.float64).float() for rid, toks in seqs.items()}
+    model = load_model(folder, dtype=dtype)
+    for steps, where in (traces.whole(seqs), traces.tail_decoded(seqs, tail=12), traces.portions(seqs, seed=seed)):
+        replay(model, steps, where, ref, dtype, 128, 16)
+    steps, where, peak = traces.mixed(seqs, seed=seed, max_live=2)
+    replay(model, steps, where, ref, dtype, peak, 16)
