@@ -164,7 +164,7 @@ def replay(model, steps, where, ref, dtype, max_tokens, page, graphs=True):
 @pytest.mark.parametrize("name", list(CONFIGS))
 @pytest.mark.parametrize("schedule", ["whole", "tail", "portions", "mixed", "mixed7"])
 def test_schedules_match_plain(folders, name, dtype, schedule):
-    """Whole prompts; prefill then token-by-token decoding (through captured steps); portions down to two tokens; mixed
+    """Whole prompts; prefill then token-by-token decoding (120 tokens, through captured steps); portions down to two tokens; mixed
     batches of unequal requests in a pool so small that pages and state slots are used again."""
     page = CONFIGS[name]["page"]
     seqs, ref, model = sequences(name), plain_logits(folders[name], name, dtype), engine_model(folders[name], name, dtype)
@@ -172,7 +172,7 @@ def test_schedules_match_plain(folders, name, dtype, schedule):
     if schedule == "whole":
         steps, where = traces.whole(seqs)
     elif schedule == "tail":
-        steps, where = traces.tail_decoded(seqs, tail=60)  # long enough to cross chunk edges and pages while decoding
+        steps, where = traces.tail_decoded(seqs, tail=120)  # long decoding: across chunk edges, pages and the convolutions' reach
     elif schedule == "portions":
         steps, where = traces.portions(seqs, seed=1)
     else:
