@@ -73,6 +73,12 @@ class CacheStorage:
                 self.views.append(StateView(t))
             else:
                 self.views.append(None)
+        # state that belongs to the model and to no layer (``model.state_needs``: name -> StateNeed)
+        self.model_state: dict[str, torch.Tensor] = {}
+        for name, need in getattr(model, "state_needs", {}).items():
+            t = torch.zeros((num_slots, *need.shape), dtype=need.dtype, device=device)
+            self.states.append(t)
+            self.model_state[name] = t
 
     def reset_slot(self, slot: int) -> None:
         """A newly admitted request starts from zero state."""

@@ -17,11 +17,13 @@ from typing import ClassVar
 
 @dataclass(frozen=True)
 class RMSNormSpec:
-    """y = w * x / sqrt(mean(x^2) + eps) over the last axis."""
+    """y = w * x / sqrt(mean(x^2) + eps) over the last axis.  ``unit_offset``: the stored weight lies around zero and the
+    factor is 1 + w, formed in 32-bit."""
 
     kind: ClassVar[str] = "rmsnorm"
     dim: int
     eps: float
+    unit_offset: bool = False
 
 
 @dataclass(frozen=True)
@@ -29,12 +31,16 @@ class RopeSpec:
     """Rotary position encoding over the first ``rotary_dim`` elements of a head; pair j is elements j and
     j + rotary_dim/2 (``interleaved``: 2j and 2j + 1).  ``scaling`` is None or the llama3 frequency scaling as
     (factor, low_freq_factor, high_freq_factor, original_max_position_embeddings).  ``cos_sin_factor`` multiplies
-    cosine and sine."""
+    cosine and sine.  ``yarn`` is None or (factor, original, fast, slow): with d(t) = rotary_dim ln(original / (2 pi t)) /
+    (2 ln theta), lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)), rotary_dim - 1) and ramp_j = clamp((j - lo) /
+    max(hi - lo, 0.001), 0, 1), pair j turns at f_j / factor * ramp_j + f_j (1 - ramp_j), and cosine and sine are
+    multiplied by 0.1 ln(factor) + 1 (on top of ``cos_sin_factor``)."""
 
     kind: ClassVar[str] = "rope"
     rotary_dim: int
     theta: float
     scaling: tuple[float, float, float, int] | None = None
+    yarn: tuple[float, float, float, float] | None = None
     max_positions: int | None = None  # None = unbounded
     interleaved: bool = False
     cos_sin_factor: float = 1.0
@@ -66,6 +72,18 @@ class AttentionSpec:
     sink: bool = False  # the soft-max's denominator holds one more term of score 0, which has no value
     own_kv: bool = True  # False: no key/value projections; the layer reads the cache of the run-order entry it names
     names: tuple[str, str, str, str] = ("q_proj.weight", "k_proj.weight", "v_proj.weight", "o_proj.weight")  # after the prefix
+    bias: bool = False  # the four projections have biases, named as their matrices plus ``bias_suffix``
+    bias_suffix: str = ".b"
+    # q (and k) pass an RMS norm over the WHOLE projection, all heads at once, with a weight per channel and this eps;
+    # the weights are named as the q and k matrices plus ``whole_norm_suffix``
+    whole_norm_eps: float | None = None
+    whole_norm_suffix: str = ".norm"
+    slope_exp: float = 0.0  # > 0: head h of H loses 2^(-slope_exp (h + 1) / H) * (query position - key position) from its score
+    # values across layers: "source" keeps this layer's values of the step's tokens for later layers; "mix" turns this
+    # layer's values into (1 - m) v + m v_source before they are cached, m one stored value named ``value_mix_name``
+    # (a "source" layer may hold that tensor too; it is not read)
+    value_mix: str = ""
+    value_mix_name: str = "vmix"
 
     @property
     def v_dim(self) -> int:
@@ -74,7 +92,32 @@ class AttentionSpec:
     @property
     def general(self) -> bool:
         return bool(self.value_dim not in (0, self.head_dim) or self.qk_norm_eps is not None or self.score_cap or self.chunk or self.sink
-                    or not self.own_kv)
+                    or not self.own_kv or self.bias or self.whole_norm_eps is not None or self.slope_exp or self.value_mix)
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Soft-max attention whose keys and values come from one cached latent per token.  With h the input:
+    c_q = norm(W_dq h); q = W_uq c_q, per head [dim unrotated | rot rotated];  W_dkv h = [latent | rot]: c = norm(first part),
+    the rest is one rotated key part for all heads;  per head k = [W_uk c | rotated part], v = W_uv c;
+    score = q . k * softmax_scale over the last ``window`` positions (0: all);  head outputs times sigmoid(W_g h) per head
+    if ``gate``;  then W_o.  The two norms are RMS norms with plain weights.  Only c and the rotated part are cached."""
+
+    kind: ClassVar[str] = "latent_attention"
+    hidden: int
+    heads: int
+    head_dim: int  # unrotated query/key channels of a head
+    rot_dim: int  # rotated ones
+    value_dim: int
+    q_rank: int
+    kv_rank: int
+    position: object  # a RopeSpec over rot_dim channels
+    softmax_scale: float
+    norm_eps: float
+    window: int = 0
+    gate: bool = True
+    # after the prefix: W_dq, its norm, W_uq, W_dkv, its norm, W_uk, W_uv, W_g, W_o
+    names: tuple = ("dq", "dq.norm", "uq", "dkv", "dkv.norm", "uk", "uv", "g", "o")
 
 
 @dataclass(frozen=True)
@@ -110,11 +153,15 @@ class DenseFFSpec:
 
 @dataclass(frozen=True)
 class SwiGLUSpec:
-    """down(silu(gate(x)) * up(x)), dense, no bias."""
+    """down(silu(gate(x)) * up(x)), dense.  ``bias``: the three projections have biases, named as their matrices plus
+    ``bias_suffix``.  ``names``: the three matrices after the prefix."""
 
     kind: ClassVar[str] = "swiglu"
     hidden: int
     intermediate: int
+    bias: bool = False
+    names: tuple[str, str, str] = ("gate_proj.weight", "up_proj.weight", "down_proj.weight")
+    bias_suffix: str = ".b"
 
 
 @dataclass(frozen=True)
@@ -142,7 +189,8 @@ class StreamBlockSpec:
     (hyper-connections).  For sublayer q (the mixer, then the feed-forward, which may be None):
         u = sum_s in_q[s] x_s;  y = sublayer(norm_q(u));  x_t <- sum_s mix_q[s, t] x_s + mult * out_q[t] * y   (all t at once)
     with the tensors ``prefix + hc_names[q] + "in" | "out" | "mix"``.  ``streams`` = 0: one stream and no such tensors,
-    x <- x + mult * sublayer(norm(x))."""
+    x <- x + mult * sublayer(norm(x)).  ``mixer_post_norm`` / ``ffn_post_norm`` (norm specs or None): a second norm behind
+    the sublayer, y = post_norm(sublayer(norm(u))), in 32-bit on the way into the streams."""
 
     kind: ClassVar[str] = "streams"
     prefix: str
@@ -157,6 +205,10 @@ class StreamBlockSpec:
     ffn_norm_name: str = "norm2"
     ffn_prefix: str = "mlp."
     hc_names: tuple[str, str] = ("hc1.", "hc2.")
+    mixer_post_norm: object | None = None
+    ffn_post_norm: object | None = None
+    mixer_post_norm_name: str = "norm1b"
+    ffn_post_norm_name: str = "norm2b"
 
 
 @dataclass(frozen=True)
@@ -168,6 +220,18 @@ class LayerCall:
 
     layer: int
     cache_from: int | None = None
+
+
+@dataclass(frozen=True)
+class PairEmbeddingSpec:
+    """A second embedding table, added to the first: row (previous token * mul_prev + token * mul_cur) mod buckets, and
+    row ``buckets`` (the last of its buckets + 1 rows) for a sequence's first token.  The previous token of a request is
+    kept in its state slot between steps."""
+
+    name: str  # tensor name of the [buckets + 1, hidden] table
+    buckets: int
+    mul_prev: int
+    mul_cur: int
 
 
 @dataclass(frozen=True)
@@ -192,6 +256,7 @@ class ModelSpec:
     # tensor-name prefixes that a checkpoint may hold although the model reads nothing under them (the tensors of a
     # sublayer that a layer does not have); anything else that is unexpected is an error
     unread_prefixes: tuple[str, ...] = field(default_factory=tuple)
+    pair_embedding: PairEmbeddingSpec | None = None  # models that carry 32-bit streams only
 
     def __post_init__(self) -> None:
         for pos, call in enumerate(self.run_order):

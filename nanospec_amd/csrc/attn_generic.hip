@@ -8,7 +8,8 @@
 // Options that the reference's attention does not have, each off at 0: ``chunk`` (a query also sees no key before the
 // start of its own chunk, floor(p / chunk) * chunk, chunks counted from position 0), ``cap`` (a score s, after the
 // scale, becomes cap * tanh(s / cap)), ``sink`` (the soft-max's denominator holds one more term of score 0 that has no
-// value), and values of another size ``vd`` than the keys' ``hd``.
+// value), values of another size ``vd`` than the keys' ``hd``, and ``slope_exp`` (a bias by distance: head h of H loses
+// 2^(-slope_exp (h + 1) / H) * (p - key) from its score, after the cap).
 // Query head h reads key/value head h / (heads / kv_heads).    (reference: model/attention.py:33)
 // K pages: [page][kv head][token][hd];  V pages: [page][kv head][vd][token].
 #include "common.h"
@@ -21,7 +22,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
     T* __restrict__ out, const T* __restrict__ q, int q_stride, const T* __restrict__ k_cache,
     const T* __restrict__ v_cache, const int* __restrict__ token_req, const int* __restrict__ positions,
     const int* __restrict__ block_table, int table_stride, int heads, int kv_heads, int hd, int vd, int page_size, float scale,
-    int window, int chunk, float cap, int sink) {
+    int window, int chunk, float cap, int sink, float slope_exp) {
   extern __shared__ float smem[];  // q_s[hd] | p_s[AG_THREADS] | scratch[16]
   float* q_s = smem;
   float* p_s = smem + hd;
@@ -36,6 +37,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
   int lo = window > 0 ? max(0, pos - window + 1) : 0;
   if (chunk > 0) lo = max(lo, pos / chunk * chunk);
   const float inv_cap = cap > 0.f ? 1.f / cap : 0.f;
+  const float slope = slope_exp > 0.f ? exp2f(-slope_exp * (float)(h + 1) / (float)heads) : 0.f;
   float m = -INFINITY, l = 0.f;
   float acc[AG_MAX_VD / AG_THREADS] = {};  // channels tid, tid + 256, ... of the output
   for (int c0 = (lo / AG_THREADS) * AG_THREADS; c0 <= pos; c0 += AG_THREADS) {
@@ -48,6 +50,7 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
       float dot = 0.f;
       for (int d = 0; d < hd; ++d) dot = fmaf(q_s[d], to_f(kr[d]), dot);
       s = cap > 0.f ? cap * tanhf(dot * inv_cap) : dot;
+      s -= slope * (float)(pos - key);
     }
     const float m_new = fmaxf(m, block_max(s, scratch));
     const float p = valid ? expf(s - m_new) : 0.f;
@@ -82,19 +85,19 @@ __global__ __launch_bounds__(AG_THREADS) void attn_generic_kernel(
 extern "C" int ns_attn_generic(void* out, const void* q, int q_stride, const void* k_cache, const void* v_cache,
                                const int* token_req, const int* positions, const int* block_table, int table_stride,
                                int n_tokens, int heads, int kv_heads, int hd, int vd, int page_size, float scale, int window,
-                               int chunk, float cap, int sink, int dtype, hipStream_t stream) {
+                               int chunk, float cap, int sink, float slope_exp, int dtype, hipStream_t stream) {
   if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || heads % kv_heads || hd <= 0 || hd > 1024 || vd <= 0 || vd > AG_MAX_VD || page_size <= 0 ||
-      window < 0 || chunk < 0 || cap < 0.f)
+      window < 0 || chunk < 0 || cap < 0.f || slope_exp < 0.f)
     return NS_ERR_BAD_ARG;
   if (heads > 65535) return NS_ERR_BAD_ARG;
   dim3 grid(n_tokens, heads);
   const size_t smem = (size_t)(hd + AG_THREADS + 16) * sizeof(float);
   if (dtype == NS_DTYPE_F32)
     attn_generic_kernel<float><<<grid, AG_THREADS, smem, stream>>>((float*)out, (const float*)q, q_stride, (const float*)k_cache,
-        (const float*)v_cache, token_req, positions, block_table, table_stride, heads, kv_heads, hd, vd, page_size, scale, window, chunk, cap, sink);
+        (const float*)v_cache, token_req, positions, block_table, table_stride, heads, kv_heads, hd, vd, page_size, scale, window, chunk, cap, sink, slope_exp);
   else if (dtype == NS_DTYPE_BF16)
     attn_generic_kernel<bf16_t><<<grid, AG_THREADS, smem, stream>>>((bf16_t*)out, (const bf16_t*)q, q_stride, (const bf16_t*)k_cache,
-        (const bf16_t*)v_cache, token_req, positions, block_table, table_stride, heads, kv_heads, hd, vd, page_size, scale, window, chunk, cap, sink);
+        (const bf16_t*)v_cache, token_req, positions, block_table, table_stride, heads, kv_heads, hd, vd, page_size, scale, window, chunk, cap, sink, slope_exp);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();
@@ -157,6 +160,82 @@ extern "C" int ns_unit_kv_write(void* qkv, int stride, const int* positions, con
   else if (dtype == NS_DTYPE_BF16)
     unit_kv_write_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)qkv, stride, positions, token_req, block_table, table_stride,
                                                                 (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, vd, page_size, eps, own_kv, vec_blocks);
+  else
+    return NS_ERR_UNSUPPORTED;
+  return ns_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// The same place in a layer whose projections carry biases, whose queries and keys pass an RMS norm over the WHOLE
+// projection (all heads at once) with a weight per channel, and whose values may be mixed with the values that an earlier
+// layer made for the same token:
+//   q <- (q + bq) / sqrt(mean((q + bq)^2 over heads*hd) + eps) * qw         (in place)
+//   k <- likewise over kv_heads*hd with kw                                   (into the K pages)
+//   v <- v + bv;  v <- (1 - lambda) v + lambda v_other  if v_other is given   (into the V pages; also to v_keep if given)
+// ``bias`` [heads*hd + kv_heads*(hd + vd)], ``qw``, ``kw`` and ``lambda`` (one value) may each be null.  One workgroup a token.
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void whole_norm_kv_write_kernel(
+    T* __restrict__ qkv, int stride, const T* __restrict__ bias, const T* __restrict__ qw, const T* __restrict__ kw,
+    const T* __restrict__ lambda, const T* __restrict__ v_other, int v_other_stride, T* __restrict__ v_keep, int v_keep_stride,
+    const int* __restrict__ positions, const int* __restrict__ token_req, const int* __restrict__ block_table, int table_stride,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, int heads, int kv_heads, int hd, int vd, int page_size, float eps) {
+  __shared__ float scratch[16];
+  const int t = blockIdx.x;
+  T* row = qkv + (size_t)t * stride;
+  const int nq = heads * hd, nk = kv_heads * hd, nv = kv_heads * vd;
+  const int pos = positions[t];
+  const int page = block_table[(size_t)token_req[t] * table_stride + pos / page_size];
+  const int slot = pos % page_size;
+  float fq = 1.f, fk = 1.f;
+  if (qw) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < nq; i += blockDim.x) {
+      const float v = to_f(row[i]) + (bias ? to_f(bias[i]) : 0.f);
+      ss = fmaf(v, v, ss);
+    }
+    fq = 1.f / sqrtf(block_sum(ss, scratch) / (float)nq + eps);
+  }
+  if (kw) {
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+      const float v = to_f(row[nq + i]) + (bias ? to_f(bias[nq + i]) : 0.f);
+      ss = fmaf(v, v, ss);
+    }
+    fk = 1.f / sqrtf(block_sum(ss, scratch) / (float)nk + eps);
+  }
+  for (int i = threadIdx.x; i < nq; i += blockDim.x) {
+    const float v = to_f(row[i]) + (bias ? to_f(bias[i]) : 0.f);
+    row[i] = from_f<T>(qw ? v * fq * to_f(qw[i]) : v);
+  }
+  for (int i = threadIdx.x; i < nk; i += blockDim.x) {
+    const float v = to_f(row[nq + i]) + (bias ? to_f(bias[nq + i]) : 0.f);
+    k_cache[(((size_t)page * kv_heads + i / hd) * page_size + slot) * hd + i % hd] = from_f<T>(kw ? v * fk * to_f(kw[i]) : v);
+  }
+  const float lam = (lambda && v_other) ? to_f(lambda[0]) : 0.f;
+  for (int i = threadIdx.x; i < nv; i += blockDim.x) {
+    float v = to_f(row[nq + nk + i]) + (bias ? to_f(bias[nq + nk + i]) : 0.f);
+    if (v_other) v = (1.f - lam) * v + lam * to_f(v_other[(size_t)t * v_other_stride + i]);
+    const T vs = from_f<T>(v);
+    if (v_keep) v_keep[(size_t)t * v_keep_stride + i] = vs;
+    v_cache[(((size_t)page * kv_heads + i / vd) * vd + i % vd) * page_size + slot] = vs;
+  }
+}
+
+extern "C" int ns_whole_norm_kv_write(void* qkv, int stride, const void* bias, const void* qw, const void* kw, const void* lambda,
+                                      const void* v_other, int v_other_stride, void* v_keep, int v_keep_stride, const int* positions,
+                                      const int* token_req, const int* block_table, int table_stride, void* k_cache, void* v_cache,
+                                      int n_tokens, int heads, int kv_heads, int hd, int vd, int page_size, float eps, int dtype,
+                                      hipStream_t stream) {
+  if (n_tokens <= 0 || heads <= 0 || kv_heads <= 0 || hd <= 0 || vd <= 0 || page_size <= 0) return NS_ERR_BAD_ARG;
+  if (dtype == NS_DTYPE_F32)
+    whole_norm_kv_write_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)qkv, stride, (const float*)bias, (const float*)qw, (const float*)kw,
+        (const float*)lambda, (const float*)v_other, v_other_stride, (float*)v_keep, v_keep_stride, positions, token_req, block_table,
+        table_stride, (float*)k_cache, (float*)v_cache, heads, kv_heads, hd, vd, page_size, eps);
+  else if (dtype == NS_DTYPE_BF16)
+    whole_norm_kv_write_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>((bf16_t*)qkv, stride, (const bf16_t*)bias, (const bf16_t*)qw, (const bf16_t*)kw,
+        (const bf16_t*)lambda, (const bf16_t*)v_other, v_other_stride, (bf16_t*)v_keep, v_keep_stride, positions, token_req, block_table,
+        table_stride, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads, hd, vd, page_size, eps);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();

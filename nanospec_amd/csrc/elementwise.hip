@@ -566,6 +566,53 @@ extern "C" int ns_silu_mul(void* out, const void* gu, int n_rows, int inter, int
   return ns_launch_status();
 }
 
+// The same for projections with biases: out[n][i] = silu(gu[n][i] + bias[i]) * (gu[n][I + i] + bias[I + i]), the sums in 32-bit.
+template <typename T>
+__global__ void silu_mul_bias_kernel(T* __restrict__ out, const T* __restrict__ gu, const T* __restrict__ bias, int inter, size_t total) {
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
+    const size_t n = e / inter;
+    const int i = (int)(e - n * inter);
+    const float g = to_f(gu[n * 2 * inter + i]) + to_f(bias[i]), u = to_f(gu[n * 2 * inter + inter + i]) + to_f(bias[inter + i]);
+    out[e] = from_f<T>(g / (1.f + expf(-g)) * u);
+  }
+}
+
+extern "C" int ns_silu_mul_bias(void* out, const void* gu, const void* bias, int n_rows, int inter, int dtype, hipStream_t stream) {
+  if (n_rows <= 0 || inter <= 0 || !bias) return NS_ERR_BAD_ARG;
+  const size_t total = (size_t)n_rows * inter;
+  const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+  if (dtype == NS_DTYPE_F32)
+    silu_mul_bias_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, (const float*)gu, (const float*)bias, inter, total);
+  else if (dtype == NS_DTYPE_BF16)
+    silu_mul_bias_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, (const bf16_t*)bias, inter, total);
+  else
+    return NS_ERR_UNSUPPORTED;
+  return ns_launch_status();
+}
+
+// out[n][i] += bias[i] in place, the sum in 32-bit.
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ out, int stride, const T* __restrict__ bias, int width, size_t total) {
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total; e += (size_t)gridDim.x * blockDim.x) {
+    const size_t n = e / width;
+    const int i = (int)(e - n * width);
+    out[n * stride + i] = from_f<T>(to_f(out[n * stride + i]) + to_f(bias[i]));
+  }
+}
+
+extern "C" int ns_add_bias(void* out, int stride, const void* bias, int n_rows, int width, int dtype, hipStream_t stream) {
+  if (n_rows <= 0 || width <= 0 || !bias) return NS_ERR_BAD_ARG;
+  const size_t total = (size_t)n_rows * width;
+  const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
+  if (dtype == NS_DTYPE_F32)
+    add_bias_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, stride, (const float*)bias, width, total);
+  else if (dtype == NS_DTYPE_BF16)
+    add_bias_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, stride, (const bf16_t*)bias, width, total);
+  else
+    return NS_ERR_UNSUPPORTED;
+  return ns_launch_status();
+}
+
 // A weight matrix back from the layout of the streaming kernels (gemm_bf16.hip:
 // wt[rt][kt][i][lane = 16 g + r][e] = w[16 rt + r][128 kt + 32 g + 8 i + e]) into plain rows [N, K], for a library product
 // over many rows where only the re-laid copy is kept.  One wave per tile of 16 rows x 128 k: four loads of a contiguous

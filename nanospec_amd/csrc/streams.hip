@@ -4,7 +4,18 @@
 //   read:   u = sum_s a[s] x_s;            h = w * u / sqrt(mean(u^2) + eps)      (h in the model's precision)
 //   write:  x_t <- sum_s M[s][t] x_s + c[t] y     for all t at once, from the old streams
 // S = 1 with a = M = 1 is the plain pre-norm residual x <- x + c y with its sum in 32-bit.
+// Two options on either side.  A norm's stored weight may lie around zero: the factor is then ``w_offset`` + w with
+// w_offset = 1, formed in 32-bit (0 leaves the weight as it is).  A sublayer's output may pass a bias and an RMS norm of
+// its own on its way into the streams (a block with norms on both sides of a sublayer):
+//   y' = (y + bias) / sqrt(mean((y + bias)^2) + eps_y) * (yw_offset + yw),   then the write with y' in place of y.
 #include "common.h"
+
+// what happens to a sublayer's output before it is written; every pointer may be null
+struct StreamPost {
+  const void* bias;  // [W] in the type of y
+  const void* yw;    // [W] in the type of y: the weight of the norm behind the sublayer
+  float y_eps, yw_offset;
+};
 
 #define NS_MAX_STREAMS 16
 
@@ -33,12 +44,66 @@ extern "C" int ns_embed_streams(float* out, const void* table, const int* ids, i
   return ns_launch_status();
 }
 
+// The same with a second table added, whose row is chosen by the token and the token before it in its sequence:
+//   row = (prev * mul_prev + token * mul_cur) mod buckets;   a sequence's first token (position 0) takes row ``buckets``.
+// The token before a step's first token of a request is part of the request's state: ``last_token`` [slots] holds the last
+// token every request has brought so far.  The workgroup of a request's first row of this step reads it and then leaves
+// the request's last token of this step there; nobody else touches that slot's word.
+template <typename T>
+__global__ void embed_pair_streams_kernel(float* __restrict__ out, const T* __restrict__ table, const T* __restrict__ pair_table,
+                                          const int* __restrict__ ids, const int* __restrict__ positions, const int* __restrict__ token_req,
+                                          const int* __restrict__ qo_indptr, const int* __restrict__ state_slots, int* __restrict__ last_token,
+                                          int hidden, int copies, float scale, int buckets, int mul_prev, int mul_cur) {
+  __shared__ int pair_row;
+  const int row = blockIdx.x;
+  const int tok = ids[row];
+  if (threadIdx.x == 0) {
+    const int b = token_req[row], first = qo_indptr[b], pos = positions[row];
+    int prev = 0;
+    if (row == first) {
+      int* word = last_token + state_slots[b];
+      prev = *word;
+      const int last = qo_indptr[b + 1] - 1;
+      if (last >= first) *word = ids[last];
+    } else {
+      prev = ids[row - 1];
+    }
+    long long v = ((long long)prev * mul_prev + (long long)tok * mul_cur) % buckets;
+    if (v < 0) v += buckets;
+    pair_row = pos == 0 ? buckets : (int)v;
+  }
+  __syncthreads();
+  const T* src = table + (size_t)tok * hidden;
+  const T* src2 = pair_table + (size_t)pair_row * hidden;
+  float* dst = out + (size_t)row * copies * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = to_f(src[i]) * scale + to_f(src2[i]);
+    for (int s = 0; s < copies; ++s) dst[(size_t)s * hidden + i] = v;
+  }
+}
+
+extern "C" int ns_embed_pair_streams(float* out, const void* table, const void* pair_table, const int* ids, const int* positions,
+                                     const int* token_req, const int* qo_indptr, const int* state_slots, int* last_token, int n_tokens,
+                                     int hidden, int copies, float scale, int buckets, int mul_prev, int mul_cur, int dtype,
+                                     hipStream_t stream) {
+  if (n_tokens <= 0 || hidden <= 0 || copies <= 0 || copies > NS_MAX_STREAMS || buckets <= 0) return NS_ERR_BAD_ARG;
+  if (dtype == NS_DTYPE_F32)
+    embed_pair_streams_kernel<float><<<n_tokens, 256, 0, stream>>>(out, (const float*)table, (const float*)pair_table, ids, positions, token_req,
+                                                                   qo_indptr, state_slots, last_token, hidden, copies, scale, buckets, mul_prev, mul_cur);
+  else if (dtype == NS_DTYPE_BF16)
+    embed_pair_streams_kernel<bf16_t><<<n_tokens, 256, 0, stream>>>(out, (const bf16_t*)table, (const bf16_t*)pair_table, ids, positions, token_req,
+                                                                    qo_indptr, state_slots, last_token, hidden, copies, scale, buckets, mul_prev, mul_cur);
+  else
+    return NS_ERR_UNSUPPORTED;
+  return ns_launch_status();
+}
+
 // One workgroup a row.  The mix u is formed twice (once for the sum of squares, once for the output) in the same order,
 // so a row costs two reads of S*W floats from cache and no scratch.  ``sum_out`` (optional): the mix itself, float.
 template <typename T>
 __global__ void stream_read_norm_kernel(T* __restrict__ out, float* __restrict__ sum_out, const float* __restrict__ x,
                                         const float* __restrict__ coeff, const T* __restrict__ w, const int* __restrict__ rows, int S,
-                                        int W, float eps) {
+                                        int W, float eps, float w_offset) {
   __shared__ float scratch[16];
   const int i = blockIdx.x;
   const size_t r = rows ? (size_t)rows[i] : (size_t)i;
@@ -57,18 +122,18 @@ __global__ void stream_read_norm_kernel(T* __restrict__ out, float* __restrict__
     float u = 0.f;
     for (int s = 0; s < S; ++s) u = fmaf(a[s], xr[(size_t)s * W + c], u);
     if (sum_out) sum_out[(size_t)i * W + c] = u;
-    if (out) out[(size_t)i * W + c] = from_f<T>(u * rinv * to_f(w[c]));
+    if (out) out[(size_t)i * W + c] = from_f<T>(u * rinv * (w_offset + to_f(w[c])));
   }
 }
 
 extern "C" int ns_stream_read_norm(void* out, float* sum_out, const float* x, const float* coeff, const void* w, const int* rows,
-                                   int n, int S, int W, float eps, int dtype, hipStream_t stream) {
+                                   int n, int S, int W, float eps, float w_offset, int dtype, hipStream_t stream) {
   if (n <= 0 || S <= 0 || S > NS_MAX_STREAMS || W <= 0) return NS_ERR_BAD_ARG;
   const int threads = W >= 1024 ? 256 : (W >= 256 ? 128 : 64);
   if (dtype == NS_DTYPE_F32)
-    stream_read_norm_kernel<float><<<n, threads, 0, stream>>>((float*)out, sum_out, x, coeff, (const float*)w, rows, S, W, eps);
+    stream_read_norm_kernel<float><<<n, threads, 0, stream>>>((float*)out, sum_out, x, coeff, (const float*)w, rows, S, W, eps, w_offset);
   else if (dtype == NS_DTYPE_BF16)
-    stream_read_norm_kernel<bf16_t><<<n, threads, 0, stream>>>((bf16_t*)out, sum_out, x, coeff, (const bf16_t*)w, rows, S, W, eps);
+    stream_read_norm_kernel<bf16_t><<<n, threads, 0, stream>>>((bf16_t*)out, sum_out, x, coeff, (const bf16_t*)w, rows, S, W, eps, w_offset);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();
@@ -108,6 +173,56 @@ extern "C" int ns_stream_write(float* x, const float* mix, const float* gain, co
   return ns_launch_status();
 }
 
+// The write with a bias and / or a norm of the sublayer's output before it: one workgroup a row, the row of y read twice.
+template <typename T>
+__global__ void stream_write_post_kernel(float* __restrict__ x, const float* __restrict__ mix, const float* __restrict__ gain,
+                                         const T* __restrict__ y, int y_stride, int S, int W, StreamPost post) {
+  __shared__ float m_s[NS_MAX_STREAMS * NS_MAX_STREAMS + NS_MAX_STREAMS];
+  __shared__ float scratch[16];
+  for (int i = threadIdx.x; i < S * S + S; i += blockDim.x) m_s[i] = i < S * S ? mix[i] : gain[i - S * S];
+  const size_t r = blockIdx.x;
+  const T* yr = y + r * y_stride;
+  const T* bias = (const T*)post.bias;
+  const T* yw = (const T*)post.yw;
+  float rinv = 1.f;
+  if (yw) {
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < W; c += blockDim.x) {
+      const float v = to_f(yr[c]) + (bias ? to_f(bias[c]) : 0.f);
+      ss = fmaf(v, v, ss);
+    }
+    ss = block_sum(ss, scratch);
+    rinv = 1.f / sqrtf(ss / (float)W + post.y_eps);
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < W; c += blockDim.x) {
+    float* xr = x + r * S * W + c;
+    float old[NS_MAX_STREAMS];
+    for (int s = 0; s < S; ++s) old[s] = xr[(size_t)s * W];
+    float yv = to_f(yr[c]) + (bias ? to_f(bias[c]) : 0.f);
+    if (yw) yv = yv * rinv * (post.yw_offset + to_f(yw[c]));
+    for (int t = 0; t < S; ++t) {
+      float v = 0.f;
+      for (int s = 0; s < S; ++s) v = fmaf(m_s[s * S + t], old[s], v);
+      xr[(size_t)t * W] = fmaf(m_s[S * S + t], yv, v);
+    }
+  }
+}
+
+extern "C" int ns_stream_write_post(float* x, const float* mix, const float* gain, const void* y, int y_stride, int n, int S, int W,
+                                    const void* bias, const void* yw, float y_eps, float yw_offset, int dtype, hipStream_t stream) {
+  if (n <= 0 || S <= 0 || S > NS_MAX_STREAMS || W <= 0) return NS_ERR_BAD_ARG;
+  const StreamPost post{bias, yw, y_eps, yw_offset};
+  const int threads = W >= 1024 ? 256 : (W >= 256 ? 128 : 64);
+  if (dtype == NS_DTYPE_F32)
+    stream_write_post_kernel<float><<<n, threads, 0, stream>>>(x, mix, gain, (const float*)y, y_stride, S, W, post);
+  else if (dtype == NS_DTYPE_BF16)
+    stream_write_post_kernel<bf16_t><<<n, threads, 0, stream>>>(x, mix, gain, (const bf16_t*)y, y_stride, S, W, post);
+  else
+    return NS_ERR_UNSUPPORTED;
+  return ns_launch_status();
+}
+
 // The two in one pass with 16-byte accesses, for S <= 4 streams and rows of a multiple of four up to 8,192 columns: the
 // write of one sublayer's output (``y`` given) followed by the read for the next sublayer (``coeff`` given), each
 // optional.  A thread keeps its columns of the mix u in registers between the sum of squares and the output, so a row is
@@ -116,11 +231,32 @@ template <typename T, int S, int KMAX>
 __global__ __launch_bounds__(256) void stream_step_kernel(float* __restrict__ x, const float* __restrict__ mix, const float* __restrict__ gain,
                                                           const T* __restrict__ y, int y_stride, const float* __restrict__ coeff,
                                                           const T* __restrict__ w, const int* __restrict__ rows, T* __restrict__ out,
-                                                          float* __restrict__ sum_out, int W, float eps, int store) {
+                                                          float* __restrict__ sum_out, int W, float eps, int store, float w_offset,
+                                                          StreamPost post) {
   __shared__ float scratch[16];
   const int i = blockIdx.x;
   const size_t r = rows ? (size_t)rows[i] : (size_t)i;
   float* xr = x + r * S * W;
+  const T* bias = (const T*)post.bias;
+  const T* yw = (const T*)post.yw;
+  float y_rinv = 1.f;
+  if (y && yw) {  // the norm behind the sublayer wants the row's sum of squares first
+    float ssy = 0.f;
+#pragma unroll
+    for (int k = 0; k < KMAX; ++k) {
+      const int c = (threadIdx.x + k * 256) * 4;
+      if (c < W) {
+        const T* yp = y + r * y_stride + c;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float v = to_f(yp[e]) + (bias ? to_f(bias[c + e]) : 0.f);
+          ssy = fmaf(v, v, ssy);
+        }
+      }
+    }
+    ssy = block_sum(ssy, scratch);
+    y_rinv = 1.f / sqrtf(ssy / (float)W + post.y_eps);
+  }
   float m[S][S], gn[S], a[S];
 #pragma unroll
   for (int s = 0; s < S; ++s) {
@@ -140,7 +276,12 @@ __global__ __launch_bounds__(256) void stream_step_kernel(float* __restrict__ x,
       for (int s = 0; s < S; ++s) v[s] = *reinterpret_cast<const float4*>(xr + (size_t)s * W + c);
       if (y) {
         const T* yp = y + r * y_stride + c;
-        const float4 yv = {to_f(yp[0]), to_f(yp[1]), to_f(yp[2]), to_f(yp[3])};
+        float4 yv = {to_f(yp[0]), to_f(yp[1]), to_f(yp[2]), to_f(yp[3])};
+        if (bias) yv.x += to_f(bias[c]), yv.y += to_f(bias[c + 1]), yv.z += to_f(bias[c + 2]), yv.w += to_f(bias[c + 3]);
+        if (yw) {
+          yv.x *= y_rinv * (post.yw_offset + to_f(yw[c])), yv.y *= y_rinv * (post.yw_offset + to_f(yw[c + 1]));
+          yv.z *= y_rinv * (post.yw_offset + to_f(yw[c + 2])), yv.w *= y_rinv * (post.yw_offset + to_f(yw[c + 3]));
+        }
         float4 nv[S];
 #pragma unroll
         for (int t = 0; t < S; ++t) {
@@ -178,8 +319,8 @@ __global__ __launch_bounds__(256) void stream_step_kernel(float* __restrict__ x,
       if (sum_out) *reinterpret_cast<float4*>(sum_out + (size_t)i * W + c) = u[k];
       if (out) {
         T* op = out + (size_t)i * W + c;
-        op[0] = from_f<T>(u[k].x * rinv * to_f(w[c])), op[1] = from_f<T>(u[k].y * rinv * to_f(w[c + 1]));
-        op[2] = from_f<T>(u[k].z * rinv * to_f(w[c + 2])), op[3] = from_f<T>(u[k].w * rinv * to_f(w[c + 3]));
+        op[0] = from_f<T>(u[k].x * rinv * (w_offset + to_f(w[c]))), op[1] = from_f<T>(u[k].y * rinv * (w_offset + to_f(w[c + 1])));
+        op[2] = from_f<T>(u[k].z * rinv * (w_offset + to_f(w[c + 2]))), op[3] = from_f<T>(u[k].w * rinv * (w_offset + to_f(w[c + 3])));
       }
     }
   }
@@ -187,23 +328,25 @@ __global__ __launch_bounds__(256) void stream_step_kernel(float* __restrict__ x,
 
 template <typename T, int S>
 static void stream_step_launch(float* x, const float* mix, const float* gain, const void* y, int y_stride, const float* coeff, const void* w,
-                               const int* rows, void* out, float* sum_out, int n, int W, float eps, int store, hipStream_t stream) {
+                               const int* rows, void* out, float* sum_out, int n, int W, float eps, int store, float w_offset,
+                               StreamPost post, hipStream_t stream) {
   if (W <= 2048)
-    stream_step_kernel<T, S, 2><<<n, 256, 0, stream>>>(x, mix, gain, (const T*)y, y_stride, coeff, (const T*)w, rows, (T*)out, sum_out, W, eps, store);
+    stream_step_kernel<T, S, 2><<<n, 256, 0, stream>>>(x, mix, gain, (const T*)y, y_stride, coeff, (const T*)w, rows, (T*)out, sum_out, W, eps, store, w_offset, post);
   else
-    stream_step_kernel<T, S, 8><<<n, 256, 0, stream>>>(x, mix, gain, (const T*)y, y_stride, coeff, (const T*)w, rows, (T*)out, sum_out, W, eps, store);
+    stream_step_kernel<T, S, 8><<<n, 256, 0, stream>>>(x, mix, gain, (const T*)y, y_stride, coeff, (const T*)w, rows, (T*)out, sum_out, W, eps, store, w_offset, post);
 }
 
 extern "C" int ns_stream_step(float* x, const float* mix, const float* gain, const void* y, int y_stride, const float* coeff, const void* w,
-                              const int* rows, void* out, float* sum_out, int n, int S, int W, float eps, int store, int dtype,
-                              hipStream_t stream) {
+                              const int* rows, void* out, float* sum_out, int n, int S, int W, float eps, int store, float w_offset,
+                              const void* bias, const void* yw, float y_eps, float yw_offset, int dtype, hipStream_t stream) {
+  const StreamPost post{bias, yw, y_eps, yw_offset};
   if (n <= 0 || S <= 0 || S > 4 || W <= 0 || W > 8192 || W % 4 || (!y && !coeff)) return NS_ERR_BAD_ARG;
   if (y && (!mix || !gain)) return NS_ERR_BAD_ARG;
   if (y && rows && store) return NS_ERR_BAD_ARG;  // a write that is kept covers every row
   if (dtype != NS_DTYPE_F32 && dtype != NS_DTYPE_BF16) return NS_ERR_UNSUPPORTED;
 #define NS_STEP(SS)                                                                                                                  \
-  if (dtype == NS_DTYPE_F32) stream_step_launch<float, SS>(x, mix, gain, y, y_stride, coeff, w, rows, out, sum_out, n, W, eps, store, stream); \
-  else stream_step_launch<bf16_t, SS>(x, mix, gain, y, y_stride, coeff, w, rows, out, sum_out, n, W, eps, store, stream)
+  if (dtype == NS_DTYPE_F32) stream_step_launch<float, SS>(x, mix, gain, y, y_stride, coeff, w, rows, out, sum_out, n, W, eps, store, w_offset, post, stream); \
+  else stream_step_launch<bf16_t, SS>(x, mix, gain, y, y_stride, coeff, w, rows, out, sum_out, n, W, eps, store, w_offset, post, stream)
   switch (S) {
     case 1: NS_STEP(1); break;
     case 2: NS_STEP(2); break;

@@ -83,8 +83,12 @@ class StepContext:
     """Device views of one step's batch plus the arena; handed to every part."""
 
     def __init__(self, layout: BatchLayout, dev_buf: torch.Tensor, arena, max_position: int, max_kv_len: int, captured: bool = False,
-                 link_norms: bool = True, max_chunk_kv: int | None = None, pad_slot: int | None = None) -> None:
+                 link_norms: bool = True, max_chunk_kv: int | None = None, pad_slot: int | None = None, model_state: dict | None = None) -> None:
         self.layout, self.arena = layout, arena
+        # per-request state that belongs to the model and to no layer, by name: tensors [slots, ...] of the cache storage
+        self.model_state = model_state or {}
+        # buffers that live as long as the step and that layers hand to each other, by key (the model fills this in)
+        self.shared: dict = {}
         # A captured step has a fixed shape; what a batch does not fill is padding: rows that belong to a stand-in request
         # whose state slot is ``pad_slot`` (None in steps without padding).  A padding row's input may be anything (no
         # mixer tile covers the padding behind the prompt portions, so what earlier kernels left in the arena flows

@@ -84,7 +84,8 @@ class _StepGraph:
 
     def context(self, runner, arena) -> StepContext:
         return StepContext(self.layout, self.dev_buf, arena, link_norms=runner.link_norms, max_position=0,
-                           max_kv_len=self.width * runner.page_size, captured=True, pad_slot=runner.manager.get(PAD_REQUEST).slot)
+                           max_kv_len=self.width * runner.page_size, captured=True, pad_slot=runner.manager.get(PAD_REQUEST).slot,
+                           model_state=getattr(runner.storage, "model_state", None))
 
 
 class ModelRunner:
@@ -265,7 +266,7 @@ class ModelRunner:
         self.arena.reset()
         chunk_kv = max((s + n for s, n in zip(starts, lens) if n != 1), default=0)
         ctx = StepContext(layout, self._dev, self.arena, max_position=max_kv - 1, max_kv_len=max_kv, link_norms=self.link_norms,
-                          max_chunk_kv=chunk_kv)
+                          max_chunk_kv=chunk_kv, model_state=getattr(self.storage, "model_state", None))
         resid, delta = self.model.forward_hidden(ctx, self.storage.views)
         if not n_want:
             return None

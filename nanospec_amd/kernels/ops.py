@@ -667,10 +667,11 @@ def _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim, v_dim: int 
 
 def attention_generic(q, out, k_cache, v_cache, token_req, positions, block_table, heads: int, kv_heads: int, head_dim: int,
                       scale: float, window: int = 0, v_dim: int | None = None, chunk: int = 0, cap: float = 0.0,
-                      sink: bool = False) -> torch.Tensor:
+                      sink: bool = False, slope_exp: float = 0.0) -> torch.Tensor:
     """Attention of every token's query over its request's pages; any key and value size up to 1024, either
     dtype.  ``chunk`` > 0: a query sees no key before the start of its own chunk of positions; ``cap`` > 0: scores become
-    cap * tanh(score / cap); ``sink``: one more term of score 0 without a value in the soft-max's denominator."""
+    cap * tanh(score / cap); ``sink``: one more term of score 0 without a value in the soft-max's denominator;
+    ``slope_exp`` > 0: head h of H loses 2^(-slope_exp (h + 1) / H) times its distance to the key from every score."""
     v_dim = head_dim if v_dim is None else v_dim
     page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim, v_dim)
     _i32(token_req, "token_req"), _i32(positions, "positions"), _i32(block_table, "block_table")
@@ -680,7 +681,7 @@ def attention_generic(q, out, k_cache, v_cache, token_req, positions, block_tabl
     _check(build.core().ns_attn_generic(_ptr(out), _ptr(q), c_int(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(token_req),
                                         _ptr(positions), _ptr(block_table), c_int(block_table.stride(0)), c_int(n), c_int(heads),
                                         c_int(kv_heads), c_int(head_dim), c_int(v_dim), c_int(page), c_float(scale), c_int(window),
-                                        c_int(chunk), c_float(cap), c_int(1 if sink else 0), c_int(_dtype_code(q)), _stream()),
+                                        c_int(chunk), c_float(cap), c_int(1 if sink else 0), c_float(slope_exp), c_int(_dtype_code(q)), _stream()),
            "attention_generic")
     return out
 
@@ -793,8 +794,8 @@ def embed_streams(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, sca
 
 
 def stream_read_norm(x: torch.Tensor, coeff: torch.Tensor, weight: torch.Tensor, eps: float, rows: torch.Tensor | None = None,
-                     out: torch.Tensor | None = None, sum_out: torch.Tensor | None = None) -> torch.Tensor:
-    """u = sum_s coeff[s] x[r, s, :] with r = rows[i] (or i); out[i] = weight * u / sqrt(mean(u^2) + eps) in the weight's dtype.
+                     out: torch.Tensor | None = None, sum_out: torch.Tensor | None = None, w_offset: float = 0.0) -> torch.Tensor:
+    """u = sum_s coeff[s] x[r, s, :] with r = rows[i] (or i); out[i] = (w_offset + weight) * u / sqrt(mean(u^2) + eps) in the weight's dtype.
     ``x`` float32 [tokens, S, W]; ``sum_out`` (float32 [n, W], optional) also receives u."""
     _f32(x, "x"), _f32(coeff, "coeff")
     _gpu(weight, rows, out, sum_out)
@@ -811,14 +812,34 @@ def stream_read_norm(x: torch.Tensor, coeff: torch.Tensor, weight: torch.Tensor,
     if sum_out is not None and (_f32(sum_out, "sum_out").shape != (n, W)):
         raise KernelRefused("stream_read_norm: sum_out must be float32 [rows, W]")
     _check(build.core().ns_stream_read_norm(_ptr(out), _ptr(sum_out), _ptr(x), _ptr(coeff), _ptr(weight), _ptr(rows), c_int(n), c_int(S),
-                                            c_int(W), c_float(eps), c_int(_dtype_code(weight)), _stream()), "stream_read_norm")
+                                            c_int(W), c_float(eps), c_float(w_offset), c_int(_dtype_code(weight)), _stream()), "stream_read_norm")
     return out
 
 
-def stream_write(x: torch.Tensor, mix: torch.Tensor, gain: torch.Tensor, y: torch.Tensor) -> None:
-    """In place, all streams at once from the old ones: x[r, t, :] = sum_s mix[s, t] x[r, s, :] + gain[t] * y[r, :]."""
+def _post_args(post: "PostNorm | None", y: torch.Tensor, W: int, what: str):
+    """-> (bias, weight, eps, offset) as the kernels take them."""
+    if post is None:
+        return _ptr(None), _ptr(None), c_float(0.0), c_float(0.0)
+    for t in (post.bias, post.weight):
+        if t is not None and (not t.is_cuda or t.shape != (W,) or not t.is_contiguous() or t.dtype != y.dtype):
+            raise KernelRefused(f"{what}: the bias and the norm weight behind a sublayer are [{W}] in the dtype of its output")
+    return _ptr(post.bias), _ptr(post.weight), c_float(post.eps), c_float(post.offset)
+
+
+def stream_write(x: torch.Tensor, mix: torch.Tensor, gain: torch.Tensor, y: torch.Tensor, post: "PostNorm | None" = None) -> None:
+    """In place, all streams at once from the old ones: x[r, t, :] = sum_s mix[s, t] x[r, s, :] + gain[t] * y[r, :]; with
+    ``post``, y first passes a bias and an RMS norm of its own (``PostNorm``)."""
     _f32(x, "x"), _f32(mix, "mix"), _f32(gain, "gain")
     _gpu(y)
+    if post is not None:
+        if x.dim() != 3 or mix.shape != (x.shape[1], x.shape[1]) or gain.shape != (x.shape[1],) or x.shape[1] > MAX_STREAMS:
+            raise KernelRefused("stream_write: x is [tokens, S, W], mix [S, S] (from, to), gain [S]")
+        if y.dim() != 2 or y.shape != (x.shape[0], x.shape[2]) or y.stride(1) != 1:
+            raise KernelRefused("stream_write: y must be [tokens, W]")
+        _check(build.core().ns_stream_write_post(_ptr(x), _ptr(mix), _ptr(gain), _ptr(y), c_int(y.stride(0)), c_int(x.shape[0]), c_int(x.shape[1]),
+                                                 c_int(x.shape[2]), *_post_args(post, y, x.shape[2], "stream_write"), c_int(_dtype_code(y)),
+                                                 _stream()), "stream_write")
+        return
     if x.dim() != 3 or mix.shape != (x.shape[1], x.shape[1]) or gain.shape != (x.shape[1],) or x.shape[1] > MAX_STREAMS:
         raise KernelRefused("stream_write: x is [tokens, S, W], mix [S, S] (from, to), gain [S]")
     if y.dim() != 2 or y.shape != (x.shape[0], x.shape[2]) or y.stride(1) != 1:
@@ -830,17 +851,26 @@ def stream_write(x: torch.Tensor, mix: torch.Tensor, gain: torch.Tensor, y: torc
 STEP_MAX_STREAMS, STEP_MAX_WIDTH = 4, 8192  # what the one-pass kernel of ``stream_step`` takes (rows of a multiple of four columns)
 
 
+class PostNorm:
+    """What a sublayer's output y passes before it is written into a 32-bit stream: a bias (the sublayer's last projection's,
+    left to this place), then an RMS norm, (y + bias) / sqrt(mean((y + bias)^2) + eps) * (offset + weight), all in 32-bit.
+    Either may be None."""
+
+    def __init__(self, bias: torch.Tensor | None = None, weight: torch.Tensor | None = None, eps: float = 0.0, offset: float = 0.0) -> None:
+        self.bias, self.weight, self.eps, self.offset = bias, weight, eps, offset
+
+
 class PendingWrite:
     """A sublayer's output on its way into a 32-bit stream: x_t <- sum_s mix[s, t] x_s + gain[t] * y, not done yet.
-    ``stream_step`` does it in the same pass as the next read."""
+    ``stream_step`` does it in the same pass as the next read.  ``post``: what y passes first (``PostNorm``)."""
 
-    def __init__(self, y: torch.Tensor, mix: torch.Tensor, gain: torch.Tensor) -> None:
-        self.y, self.mix, self.gain = y, mix, gain
+    def __init__(self, y: torch.Tensor, mix: torch.Tensor, gain: torch.Tensor, post: "PostNorm | None" = None) -> None:
+        self.y, self.mix, self.gain, self.post = y, mix, gain, post
 
 
 def stream_step(x: torch.Tensor, pending: "PendingWrite | None", coeff: torch.Tensor | None = None, weight: torch.Tensor | None = None,
                 eps: float = 0.0, rows: torch.Tensor | None = None, out: torch.Tensor | None = None, sum_out: torch.Tensor | None = None,
-                store: bool = True) -> torch.Tensor | None:
+                store: bool = True, w_offset: float = 0.0) -> torch.Tensor | None:
     """``stream_write`` of ``pending`` (if any) and then ``stream_read_norm`` with ``coeff`` and ``weight`` (if any), in one
     pass over the rows where the sizes allow it, in two kernels otherwise.  With ``rows`` the read is of those rows only,
     and a pending write is then done on the fly for them and not kept (``store`` must be False): for the last read of a step."""
@@ -850,8 +880,8 @@ def stream_step(x: torch.Tensor, pending: "PendingWrite | None", coeff: torch.Te
     one_pass = S <= STEP_MAX_STREAMS and W <= STEP_MAX_WIDTH and W % 4 == 0
     if not one_pass:
         if pending is not None:  # (kept whatever ``store`` says: keeping it harms nobody)
-            stream_write(x, pending.mix, pending.gain, pending.y)
-        return stream_read_norm(x, coeff, weight, eps, rows=rows, out=out, sum_out=sum_out) if coeff is not None else None
+            stream_write(x, pending.mix, pending.gain, pending.y, pending.post)
+        return stream_read_norm(x, coeff, weight, eps, rows=rows, out=out, sum_out=sum_out, w_offset=w_offset) if coeff is not None else None
     _f32(x, "x")
     y = None
     if pending is not None:
@@ -880,8 +910,158 @@ def stream_step(x: torch.Tensor, pending: "PendingWrite | None", coeff: torch.Te
         return None
     _check(build.core().ns_stream_step(_ptr(x), _ptr(pending.mix if pending else None), _ptr(pending.gain if pending else None), _ptr(y),
                                        c_int(y.stride(0) if y is not None else 0), _ptr(coeff), _ptr(weight), _ptr(rows), _ptr(out),
-                                       _ptr(sum_out), c_int(n), c_int(S), c_int(W), c_float(eps), c_int(1 if store else 0),
+                                       _ptr(sum_out), c_int(n), c_int(S), c_int(W), c_float(eps), c_int(1 if store else 0), c_float(w_offset),
+                                       *_post_args(pending.post if pending else None, y, W, "stream_step"),
                                        c_int(BF16 if dtype == torch.bfloat16 else F32), _stream()), "stream_step")
+    return out
+
+
+def embed_pair_streams(table: torch.Tensor, pair_table: torch.Tensor, ids, positions, token_req, qo_indptr, state_slots, last_token: torch.Tensor,
+                       out: torch.Tensor, scale: float, buckets: int, mul_prev: int, mul_cur: int) -> torch.Tensor:
+    """``embed_streams`` plus a row of a second table chosen by the token and the one before it in its sequence:
+    row (prev * mul_prev + token * mul_cur) mod buckets, and row ``buckets`` for a sequence's first token (position 0).
+    ``last_token`` int32 [slots, 1]: every request's last token so far; read for a request's first row of the step and left
+    holding its last token of the step."""
+    _gpu(table, pair_table, ids, positions, token_req, qo_indptr, state_slots, last_token)
+    for name, t in (("ids", ids), ("positions", positions), ("token_req", token_req), ("qo_indptr", qo_indptr), ("state_slots", state_slots),
+                    ("last_token", last_token)):
+        _i32(t, name)
+    _f32(out, "out")
+    n, hidden = ids.numel(), table.shape[1]
+    if (out.dim() != 3 or out.shape[0] != n or out.shape[2] != hidden or not 1 <= out.shape[1] <= MAX_STREAMS or not table.is_contiguous()
+            or pair_table.shape != (buckets + 1, hidden) or not pair_table.is_contiguous() or pair_table.dtype != table.dtype
+            or positions.numel() != n or token_req.numel() != n or qo_indptr.numel() != state_slots.numel() + 1):
+        raise KernelRefused(f"embed_pair_streams: out float32 [{n}, copies, {hidden}], the second table [{buckets + 1}, {hidden}]")
+    _check(build.core().ns_embed_pair_streams(_ptr(out), _ptr(table), _ptr(pair_table), _ptr(ids), _ptr(positions), _ptr(token_req),
+                                              _ptr(qo_indptr), _ptr(state_slots), _ptr(last_token), c_int(n), c_int(hidden), c_int(out.shape[1]),
+                                              c_float(scale), c_int(buckets), c_int(mul_prev), c_int(mul_cur), c_int(_dtype_code(table)),
+                                              _stream()), "embed_pair_streams")
+    return out
+
+
+def whole_norm_kv_write(qkv: torch.Tensor, positions, token_req, block_table, k_cache, v_cache, heads: int, kv_heads: int, head_dim: int,
+                        v_dim: int, eps: float, bias: torch.Tensor | None = None, q_weight: torch.Tensor | None = None,
+                        k_weight: torch.Tensor | None = None, mix: torch.Tensor | None = None, v_other: torch.Tensor | None = None,
+                        v_keep: torch.Tensor | None = None) -> None:
+    """For attention without rotation whose projections carry biases and whose queries and keys pass an RMS norm over the whole
+    projection.  A row of ``qkv`` is q [heads * head_dim], k [kv_heads * head_dim], v [kv_heads * v_dim]; ``bias`` of that
+    width is added; q (in place) and k become x / sqrt(mean(x^2 over the whole projection) + eps) * weight; v becomes
+    (1 - mix) v + mix v_other where ``v_other`` [tokens, kv_heads * v_dim] is given (``mix``: one value on the device), is
+    copied to ``v_keep`` where that is given, and k and v go into the pages of their positions."""
+    _gpu(qkv, positions, token_req, block_table, k_cache, v_cache, bias, q_weight, k_weight, mix, v_other, v_keep)
+    n = positions.numel()
+    nq, nk, nv = heads * head_dim, kv_heads * head_dim, kv_heads * v_dim
+    if qkv.dim() != 2 or qkv.shape[0] != n or qkv.shape[1] < nq + nk + nv or qkv.stride(1) != 1:
+        raise KernelRefused(f"whole_norm_kv_write: qkv must be [{n}, {nq + nk + nv}]")
+    _i32(positions, "positions"), _i32(token_req, "token_req"), _i32(block_table, "block_table")
+    if token_req.numel() != n or block_table.dim() != 2 or block_table.stride(1) != 1:
+        raise KernelRefused("whole_norm_kv_write: token_req is per token, block_table int32 [requests, pages]")
+    page = k_cache.shape[2] if k_cache.dim() == 4 else 0
+    if (k_cache.dim() != 4 or k_cache.shape[1:] != (kv_heads, page, head_dim) or v_cache.shape != (k_cache.shape[0], kv_heads, v_dim, page)
+            or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
+        raise KernelRefused("whole_norm_kv_write: cache pages do not fit heads, sizes or dtype")
+    for t, size, name in ((bias, nq + nk + nv, "bias"), (q_weight, nq, "q_weight"), (k_weight, nk, "k_weight"), (mix, 1, "mix")):
+        if t is not None and (t.numel() != size or not t.is_contiguous() or t.dtype != qkv.dtype):
+            raise KernelRefused(f"whole_norm_kv_write: {name} holds {size} values of the dtype of qkv")
+    for t, name in ((v_other, "v_other"), (v_keep, "v_keep")):
+        if t is not None and (t.dim() != 2 or t.shape != (n, nv) or t.stride(1) != 1 or t.dtype != qkv.dtype):
+            raise KernelRefused(f"whole_norm_kv_write: {name} must be [{n}, {nv}] of the dtype of qkv")
+    if v_other is not None and mix is None:
+        raise KernelRefused("whole_norm_kv_write: values of another layer come with the weight they are mixed in with")
+    _check(build.core().ns_whole_norm_kv_write(_ptr(qkv), c_int(qkv.stride(0)), _ptr(bias), _ptr(q_weight), _ptr(k_weight), _ptr(mix),
+                                               _ptr(v_other), c_int(v_other.stride(0) if v_other is not None else 0), _ptr(v_keep),
+                                               c_int(v_keep.stride(0) if v_keep is not None else 0), _ptr(positions), _ptr(token_req),
+                                               _ptr(block_table), c_int(block_table.stride(0)), _ptr(k_cache), _ptr(v_cache), c_int(n),
+                                               c_int(heads), c_int(kv_heads), c_int(head_dim), c_int(v_dim), c_int(page), c_float(eps),
+                                               c_int(_dtype_code(qkv)), _stream()), "whole_norm_kv_write")
+
+
+def silu_mul_bias(gu: torch.Tensor, bias: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[n, i] = silu(gu[n, i] + bias[i]) * (gu[n, I + i] + bias[I + i]) for gu [N, 2 I]."""
+    _gpu(gu, bias)
+    n, two_i = gu.shape
+    inter = two_i // 2
+    if two_i % 2 or not gu.is_contiguous() or bias.shape != (two_i,) or not bias.is_contiguous() or bias.dtype != gu.dtype:
+        raise KernelRefused("silu_mul_bias: gu must be contiguous [N, 2 I], bias [2 I] of its dtype")
+    if out is None:
+        out = torch.empty((n, inter), dtype=gu.dtype, device=gu.device)
+    if out.shape != (n, inter) or not out.is_contiguous() or out.dtype != gu.dtype:
+        raise KernelRefused("silu_mul_bias: out must be contiguous [N, I]")
+    _check(build.core().ns_silu_mul_bias(_ptr(out), _ptr(gu), _ptr(bias), c_int(n), c_int(inter), c_int(_dtype_code(gu)), _stream()), "silu_mul_bias")
+    return out
+
+
+def add_bias(out: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """out[n, :] += bias, in place."""
+    _gpu(out, bias)
+    if out.dim() != 2 or out.stride(1) != 1 or bias.shape != (out.shape[1],) or not bias.is_contiguous() or bias.dtype != out.dtype:
+        raise KernelRefused("add_bias: out [N, W] and bias [W] of one dtype")
+    _check(build.core().ns_add_bias(_ptr(out), c_int(out.stride(0)), _ptr(bias), c_int(out.shape[0]), c_int(out.shape[1]), c_int(_dtype_code(out)),
+                                    _stream()), "add_bias")
+    return out
+
+
+def latent_prep(proj: torch.Tensor, q_norm: torch.Tensor, c_norm: torch.Tensor, inv_freq: torch.Tensor, factor: float, positions, token_req,
+                block_table, k_cache, v_cache, q_rank: int, latent: int, rot: int, heads: int, eps: float, cq: torch.Tensor,
+                gate: torch.Tensor | None) -> None:
+    """What a latent-attention layer does to a token's row [q_rank | latent | rot | heads] of its first product: the first
+    q_rank values RMS-normed with ``q_norm`` into ``cq``; the next ``latent`` RMS-normed with ``c_norm`` and the ``rot`` behind
+    them rotated by the position (pair i, i + rot/2; ``factor`` on cosine and sine) into the K page as one key [latent + rot];
+    the normed latent also into the V page; sigmoid of the last ``heads`` values into ``gate`` (float32; ``heads`` = 0 and None for a
+    layer without gates)."""
+    _gpu(proj, q_norm, c_norm, inv_freq, positions, token_req, block_table, k_cache, v_cache, cq, gate)
+    n = positions.numel()
+    width = q_rank + latent + rot + heads
+    _i32(positions, "positions"), _i32(token_req, "token_req"), _i32(block_table, "block_table"), _f32(inv_freq, "inv_freq")
+    if (gate is None) != (heads == 0) or (gate is not None and _f32(gate, "gate").shape != (n, heads)):
+        raise KernelRefused(f"latent_prep: gate is float32 [{n}, {heads}] (None without gates)")
+    if proj.dim() != 2 or proj.shape[0] != n or proj.shape[1] < width or proj.stride(1) != 1:
+        raise KernelRefused(f"latent_prep: the projected rows must be [{n}, {width}]")
+    page = k_cache.shape[2] if k_cache.dim() == 4 else 0
+    if (k_cache.dim() != 4 or k_cache.shape[1:] != (1, page, latent + rot) or v_cache.shape != (k_cache.shape[0], 1, latent, page)
+            or k_cache.dtype != proj.dtype or v_cache.dtype != proj.dtype or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
+        raise KernelRefused("latent_prep: the pages hold one key of latent + rot channels and one value of latent channels per token")
+    if (q_norm.shape != (q_rank,) or c_norm.shape != (latent,) or q_norm.dtype != proj.dtype or c_norm.dtype != proj.dtype or not q_norm.is_contiguous()
+            or not c_norm.is_contiguous() or cq.shape != (n, q_rank) or cq.dtype != proj.dtype or not cq.is_contiguous()
+            or rot % 2 or inv_freq.numel() < max(1, rot // 2) or token_req.numel() != n or block_table.dim() != 2 or block_table.stride(1) != 1):
+        raise KernelRefused("latent_prep: norm weights, outputs or frequencies do not fit the sizes")
+    _check(build.core().ns_latent_prep(_ptr(proj), c_int(proj.stride(0)), _ptr(q_norm), _ptr(c_norm), _ptr(inv_freq), c_float(factor), _ptr(cq),
+                                       _ptr(gate), _ptr(positions), _ptr(token_req), _ptr(block_table), c_int(block_table.stride(0)),
+                                       _ptr(k_cache), _ptr(v_cache), c_int(n), c_int(q_rank), c_int(latent), c_int(rot), c_int(heads),
+                                       c_int(page), c_float(eps), c_int(_dtype_code(proj)), _stream()), "latent_prep")
+
+
+def latent_q_absorb(q: torch.Tensor, uk: torch.Tensor, inv_freq: torch.Tensor, factor: float, positions, heads: int, dim: int, rot: int,
+                    latent: int, out: torch.Tensor) -> torch.Tensor:
+    """q [tokens, heads * (dim + rot)] -> out [tokens, heads * (latent + rot)]: per head, the first ``dim`` values through
+    that head's key matrix, out[c] = sum_d q[d] uk[head * dim + d, c] (``uk`` [heads * dim, latent]), and the ``rot`` values
+    behind them rotated by the position."""
+    _gpu(q, uk, inv_freq, positions, out)
+    n = positions.numel()
+    _i32(positions, "positions"), _f32(inv_freq, "inv_freq")
+    if (q.dim() != 2 or q.shape != (n, heads * (dim + rot)) or q.stride(1) != 1 or uk.shape != (heads * dim, latent) or not uk.is_contiguous()
+            or uk.dtype != q.dtype or out.shape != (n, heads * (latent + rot)) or not out.is_contiguous() or out.dtype != q.dtype or rot % 2
+            or inv_freq.numel() < max(1, rot // 2) or dim > 2048):
+        raise KernelRefused("latent_q_absorb: q [tokens, heads * (dim + rot)], uk [heads * dim, latent], out [tokens, heads * (latent + rot)]")
+    _check(build.core().ns_latent_q_absorb(_ptr(q), c_int(q.stride(0)), _ptr(uk), _ptr(inv_freq), c_float(factor), _ptr(positions), _ptr(out),
+                                           c_int(n), c_int(heads), c_int(dim), c_int(rot), c_int(latent), c_int(_dtype_code(q)), _stream()),
+           "latent_q_absorb")
+    return out
+
+
+def latent_out(o: torch.Tensor, uv_t: torch.Tensor, gate: torch.Tensor | None, heads: int, latent: int, v_dim: int, out: torch.Tensor) -> torch.Tensor:
+    """o [tokens, heads * latent] -> out [tokens, heads * v_dim]: out[h, e] = gate[h] * sum_c o[h, c] uv_t[h, c, e]
+    (``uv_t`` [heads, latent, v_dim]; ``gate`` float32 [tokens, heads] or None)."""
+    _gpu(o, uv_t, gate, out)
+    n = o.shape[0]
+    if gate is not None:
+        _f32(gate, "gate")
+    if (o.dim() != 2 or o.shape != (n, heads * latent) or not o.is_contiguous() or uv_t.shape != (heads, latent, v_dim) or not uv_t.is_contiguous()
+            or uv_t.dtype != o.dtype or out.shape != (n, heads * v_dim) or not out.is_contiguous() or out.dtype != o.dtype
+            or (gate is not None and gate.shape != (n, heads)) or latent > 2048):
+        raise KernelRefused("latent_out: o [tokens, heads * latent], uv_t [heads, latent, v_dim], out [tokens, heads * v_dim]")
+    _check(build.core().ns_latent_out(_ptr(o), _ptr(uv_t), _ptr(gate), _ptr(out), c_int(n), c_int(heads), c_int(latent), c_int(v_dim),
+                                      c_int(_dtype_code(o)), _stream()), "latent_out")
     return out
 
 

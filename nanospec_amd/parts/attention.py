@@ -148,6 +148,21 @@ class Attention:
             raise ValueError("the rotary part of a head cannot be wider than the head")
         self.wqkv: LinearWeight | None = None
         self.wo: LinearWeight | None = None
+        self.qkv_bias = self.q_norm = self.k_norm = self.v_mix = None
+        self.out_bias: torch.Tensor | None = None  # the output projection's bias; a block may add it itself (add_out_bias=False)
+        if spec.value_mix not in ("", "source", "mix"):
+            raise ValueError(f"value_mix={spec.value_mix!r}: use '', 'source' or 'mix'")
+        if (spec.bias or spec.whole_norm_eps is not None or spec.value_mix) and not spec.own_kv:
+            raise ValueError("biases, whole-projection norms and mixed values belong to a layer with key/value projections of its own")
+        if spec.whole_norm_eps is not None and (spec.qk_norm_eps is not None or self.position.rotary_dim):
+            raise ValueError("a norm over the whole projection stands alone: no per-head unit norm and no rotation beside it")
+
+    VALUES_KEY = "attention.values"  # where a "source" layer leaves its values of the step's tokens (``ctx.shared``)
+
+    def step_buffers(self) -> dict:
+        """Buffers that live as long as a step and that layers hand to each other: key -> columns per token."""
+        s = self.spec
+        return {self.VALUES_KEY: s.kv_heads * s.v_dim} if s.value_mix else {}
 
     @property
     def _names(self):
@@ -161,6 +176,16 @@ class Attention:
         if s.own_kv:
             out[k] = ((s.kv_heads * s.head_dim, s.hidden), "linear")
             out[v] = ((s.kv_heads * s.v_dim, s.hidden), "linear")
+        if s.bias:
+            for name in (q, k, v, o):
+                out[name + s.bias_suffix] = ((out[name][0][0],), "bias")
+        if s.whole_norm_eps is not None:
+            out[q + s.whole_norm_suffix] = ((s.heads * s.head_dim,), "norm")
+            out[k + s.whole_norm_suffix] = ((s.kv_heads * s.head_dim,), "norm")
+        if s.value_mix:
+            # (a "source" layer's checkpoint holds the tensor too; it is not used there)
+            out[self.prefix + s.value_mix_name] = ((), lambda shape, gen: torch.full(shape, 0.5, device=gen.device)
+                                                   + 0.2 * torch.randn(shape, generator=gen, dtype=torch.float32, device=gen.device))
         return out
 
     def load(self, get, dtype, device, layouts: str = "both") -> None:
@@ -177,6 +202,14 @@ class Attention:
         self.position.load(get, dtype, device)
         # how the position encoding pairs channels and scales cosine and sine (the kernels' ``RopeForm``)
         self._form = dict(interleaved=bool(getattr(self.position, "interleaved", False)), factor=float(getattr(self.position, "factor", 1.0)))
+        to = lambda name: get(name).to(device=device, dtype=dtype).contiguous()
+        if s.bias:
+            self.qkv_bias = torch.cat([to(name + s.bias_suffix) for name in (q, k, v)]).contiguous()
+            self.out_bias = to(o + s.bias_suffix)
+        if s.whole_norm_eps is not None:
+            self.q_norm, self.k_norm = to(q + s.whole_norm_suffix), to(k + s.whole_norm_suffix)
+        if s.value_mix == "mix":
+            self.v_mix = to(self.prefix + s.value_mix_name).reshape(1)
         if s.general:
             # the general path: one product for what the layer projects, then norm / cache write and attention as kernels
             self.wqkv_rope = None
@@ -213,7 +246,7 @@ class Attention:
         first = self.wqkv_rope is not None or self.wqkv.links_norms(rows)
         return rows <= 16 and first and self.wo.links_norms(rows)
 
-    def forward(self, ctx, x, cache, owns_cache: bool = True, out: torch.Tensor | None = None, residual=None):
+    def forward(self, ctx, x, cache, owns_cache: bool = True, out: torch.Tensor | None = None, residual=None, add_out_bias: bool = True):
         s = self.spec
         n = x.shape[0]
         pos = self.position
@@ -222,7 +255,7 @@ class Attention:
         qkv = ctx.arena.take((n, self.wqkv.n), x.dtype)
         table = ctx.block_tables[cache.group]
         if s.general:
-            return self._forward_general(ctx, x, cache, owns_cache, out, residual, qkv, table)
+            return self._forward_general(ctx, x, cache, owns_cache, out, residual, qkv, table, add_out_bias)
         if self.wqkv_rope is not None and n <= 16 and ops.tiled_takes(x.x if isinstance(x, ops.PreNormed) else x, s.hidden):
             ops.linear_qkv_rope(x, self.wqkv_rope, qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v,
                                 s.heads, s.kv_heads, s.head_dim, pos.rotary_dim, write_kv=owns_cache, **self._form)
@@ -256,10 +289,11 @@ class Attention:
         return self.wo(att, out=out, arena=ctx.arena, plain_copy=not ctx.captured)
 
 
-    def _forward_general(self, ctx, x, cache, owns_cache, out, residual, qkv, table):
+    def _forward_general(self, ctx, x, cache, owns_cache, out, residual, qkv, table, add_out_bias=True):
         """Attention with any of the spec's options: values of another size than the keys, unit-RMS queries and keys, capped
-        scores, a chunked mask, a sink, keys and values of another layer.  The cache holds keys as the scores meet them
-        (after norm and rotation), so a layer that borrows them brings only its queries."""
+        scores, a chunked mask, a sink, keys and values of another layer, biases, a norm over the whole of q and of k, a
+        bias by distance, values mixed with an earlier layer's.  The cache holds keys as the scores meet them (after norm
+        and rotation) and values as they are read (after mixing), so a layer that borrows them brings only its queries."""
         s, pos = self.spec, self.position
         n = x.shape[0]
         if s.own_kv != bool(owns_cache):
@@ -270,13 +304,25 @@ class Attention:
         if pos.rotary_dim:
             if s.qk_norm_eps is not None or s.v_dim != s.head_dim or not s.own_kv:
                 raise ops.KernelRefused("rotation together with unit-RMS queries and keys, another value size or borrowed keys is not built")
+            if s.bias or s.value_mix:
+                raise ops.KernelRefused("rotation together with biases or mixed values is not built")
             ops.rope_kv_write(qkv, ctx.positions, ctx.token_req, table, pos.inv_freq, cache.k, cache.v, s.heads, s.kv_heads,
                               s.head_dim, pos.rotary_dim, write_kv=True, **self._form)
+        elif s.bias or s.whole_norm_eps is not None or s.value_mix:
+            if s.qk_norm_eps is not None:
+                raise ops.KernelRefused("a per-head unit norm together with biases, a whole-projection norm or mixed values is not built")
+            shared = ctx.shared.get(self.VALUES_KEY) if s.value_mix else None
+            if s.value_mix and shared is None:
+                raise ops.KernelRefused("the step holds no buffer for the values that layers hand to each other")
+            ops.whole_norm_kv_write(qkv, ctx.positions, ctx.token_req, table, cache.k, cache.v, s.heads, s.kv_heads, s.head_dim, s.v_dim,
+                                    s.whole_norm_eps or 0.0, bias=self.qkv_bias, q_weight=self.q_norm, k_weight=self.k_norm,
+                                    mix=self.v_mix, v_other=shared if s.value_mix == "mix" else None,
+                                    v_keep=shared if s.value_mix == "source" else None)
         else:
             ops.unit_kv_write(qkv, ctx.positions, ctx.token_req, table, cache.k, cache.v, s.heads, s.kv_heads, s.head_dim, s.v_dim,
                               s.qk_norm_eps, own_kv=s.own_kv)
         att = ctx.arena.take((n, s.heads * s.v_dim), x.dtype)
-        if s.v_dim == s.head_dim and ops.mfma_attention_takes(x.dtype, s.head_dim, cache.k.shape[2]):
+        if s.v_dim == s.head_dim and not s.slope_exp and ops.mfma_attention_takes(x.dtype, s.head_dim, cache.k.shape[2]):
             # bfloat16 on the matrix cores: the tile kernels honour chunks, capped scores and the sink
             for plan in launch_plans(ctx, s.heads // s.kv_heads, s.kv_heads, s.head_dim, span=s.chunk):
                 ops.attention_mfma(qkv, att, cache.k, cache.v, plan.tiles, table, s.heads, s.kv_heads, s.head_dim, s.softmax_scale,
@@ -284,10 +330,12 @@ class Attention:
                                    chunk=s.chunk, cap=s.score_cap, sink=s.sink)
         else:
             ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads, s.head_dim,
-                                  s.softmax_scale, window=s.window, v_dim=s.v_dim, chunk=s.chunk, cap=s.score_cap, sink=s.sink)
-        if residual is not None:
+                                  s.softmax_scale, window=s.window, v_dim=s.v_dim, chunk=s.chunk, cap=s.score_cap, sink=s.sink,
+                                  slope_exp=s.slope_exp)
+        if residual is not None and self.out_bias is None:
             return self.wo.into_residual(att, residual, arena=ctx.arena, plain_copy=not ctx.captured)
-        return self.wo(att, out=out, arena=ctx.arena, plain_copy=not ctx.captured)
+        y = self.wo(att, out=out if out is not None else ctx.arena.take((n, s.hidden), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)
+        return ops.add_bias(y, self.out_bias) if (self.out_bias is not None and add_out_bias) else y
 
 
 registry.register("mixer", "attention", Attention)

@@ -125,10 +125,17 @@ class StreamBlock:
         self.mixer = registry.build("mixer", spec.mixer, p + spec.mixer_prefix)
         self.ffn = registry.build("ffn", spec.ffn, p + spec.ffn_prefix) if spec.ffn is not None else None
         self.ffn_norm = registry.build("norm", spec.ffn_norm, p + spec.ffn_norm_name) if spec.ffn is not None else None
-        self.parts = tuple(x for x in (self.mixer_norm, self.mixer, self.ffn_norm, self.ffn) if x is not None)
+        # norms behind the sublayers (x <- x + post_norm(sublayer(norm(x)))), applied as the output is written into the streams
+        post = lambda given, name: registry.build("norm", given, p + name) if given is not None else None
+        self.mixer_post = post(getattr(spec, "mixer_post_norm", None), getattr(spec, "mixer_post_norm_name", ""))
+        self.ffn_post = post(getattr(spec, "ffn_post_norm", None), getattr(spec, "ffn_post_norm_name", "")) if spec.ffn is not None else None
+        self.parts = tuple(x for x in (self.mixer_norm, self.mixer, self.mixer_post, self.ffn_norm, self.ffn, self.ffn_post) if x is not None)
         for norm in (self.mixer_norm, self.ffn_norm):
             if norm is not None and not hasattr(norm, "read_streams"):
                 raise ValueError(f"a norm of kind {norm.spec.kind!r} cannot read a 32-bit stream (it has no read_streams)")
+        for norm in (self.mixer_post, self.ffn_post):
+            if norm is not None and not hasattr(norm, "behind"):
+                raise ValueError(f"a norm of kind {norm.spec.kind!r} cannot stand behind a sublayer of a 32-bit stream (it has no behind)")
         self._hc: list = []  # per sublayer: (in [S], mix [S, S], mult * out [S]) float32 on the device
 
     @property
@@ -184,6 +191,19 @@ class StreamBlock:
         limits = [n for n in limits if n is not None]
         return min(limits) if limits else None
 
+    @staticmethod
+    def _sublayer(part, post_norm, ctx, h, *cache, out):
+        """Run a sublayer.  -> (its output, what the output passes on its way into the streams: an ``ops.PostNorm`` or None).
+        A sublayer whose last projection has a bias (``out_bias``) leaves it to that place, where it is added in 32-bit."""
+        bias = getattr(part, "out_bias", None)
+        if bias is not None:
+            y = part.forward(ctx, h, *cache, out=out, add_out_bias=False)
+        else:
+            y = part.forward(ctx, h, *cache, out=out)
+        if post_norm is not None:
+            return y, post_norm.behind(bias)
+        return y, (ops.PostNorm(bias=bias) if bias is not None else None)
+
     def forward(self, ctx, resid, delta, cache, owns_cache, delta_out):
         """``resid``: float32 [tokens, S, width], updated in place.  ``delta``: None, or the ``ops.PendingWrite`` that the block
         before left (its last sublayer's output, not yet in the streams): it is written by the kernel that reads for this
@@ -198,13 +218,14 @@ class StreamBlock:
         a, mix, gain = self._hc[0]
         h = self.mixer_norm.read_streams(ctx, resid, a, out=ctx.arena.take((n, W), dtype), pending=delta)
         last = self.ffn is None
-        y = self.mixer.forward(ctx, h, cache, owns_cache, out=delta_out if last and delta_out is not None else ctx.arena.take((n, W), dtype))
-        pending = ops.PendingWrite(y, mix, gain)
+        y, post = self._sublayer(self.mixer, self.mixer_post, ctx, h, cache, owns_cache,
+                                 out=delta_out if last and delta_out is not None else ctx.arena.take((n, W), dtype))
+        pending = ops.PendingWrite(y, mix, gain, post)
         if not last:
             a, mix, gain = self._hc[1]
             h = self.ffn_norm.read_streams(ctx, resid, a, out=h, pending=pending)
-            y = self.ffn.forward(ctx, h, out=delta_out if delta_out is not None else y)
-            pending = ops.PendingWrite(y, mix, gain)
+            y, post = self._sublayer(self.ffn, self.ffn_post, ctx, h, out=delta_out if delta_out is not None else y)
+            pending = ops.PendingWrite(y, mix, gain, post)
         if delta_out is None:
             ops.stream_step(resid, pending)
             pending = None

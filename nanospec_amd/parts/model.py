@@ -23,6 +23,9 @@ def wanted_tensors(spec, layers=None) -> dict:
     """Every tensor the model reads from a checkpoint: name -> (shape, role)."""
     layers = layers if layers is not None else _build_layers(spec)
     out = {spec.embed_name: ((spec.vocab_size, spec.hidden), "embedding")}
+    pair = getattr(spec, "pair_embedding", None)
+    if pair is not None:
+        out[pair.name] = ((pair.buckets + 1, spec.hidden), "embedding")
     for layer in layers:
         out.update(layer.wanted())
     out.update(registry.build("norm", spec.final_norm, spec.final_norm_name).wanted())
@@ -31,6 +34,8 @@ def wanted_tensors(spec, layers=None) -> dict:
 
 
 class DecoderModel:
+    LAST_TOKEN = "last_token"  # model state: the last token that every request has brought so far
+
     def __init__(self, spec, config=None) -> None:
         self.spec, self.config = spec, config
         self.layers = _build_layers(spec)
@@ -47,6 +52,20 @@ class DecoderModel:
             raise ValueError(f"the blocks carry the residual stream as {sorted(forms)}, the model as {'streams' if spec.streams else 'single'}")
         if spec.streams and not hasattr(self.final_norm, "read_streams"):
             raise ValueError("the last norm cannot read a 32-bit stream (it has no read_streams)")
+        self.pair = getattr(spec, "pair_embedding", None)
+        if self.pair is not None and not spec.streams:
+            raise ValueError("a pair embedding is built for models that carry 32-bit streams")
+        self.pair_table: torch.Tensor | None = None
+        # state of fixed size per request that belongs to no layer: name -> StateNeed (the cache storage keeps a tensor
+        # [slots, *shape] for each, zeroed at admission, and the step's context hands them over as ``ctx.model_state``)
+        self.state_needs = {self.LAST_TOKEN: StateNeed((1,), torch.int32)} if self.pair is not None else {}
+        # buffers that live as long as a step and that layers hand to each other (``ctx.shared``): key -> columns per token
+        self.step_buffers: dict[str, int] = {}
+        for layer in self.layers:
+            for part in getattr(layer, "parts", ()):
+                for key, cols in getattr(part, "step_buffers", dict)().items():
+                    if self.step_buffers.setdefault(key, cols) != cols:
+                        raise ValueError(f"two layers want the step's buffer {key!r} with {self.step_buffers[key]} and {cols} columns")
         self._ones: torch.Tensor | None = None
         # for tests and debugging: called as layer_probe(run-order entry, float32 [tokens, hidden]) with the sum of the
         # streams after every entry (eager steps of models that carry 32-bit streams)
@@ -101,6 +120,8 @@ class DecoderModel:
             else:
                 layer.load(get, dtype, device)
         self.final_norm.load(get, dtype, device)
+        if self.pair is not None:
+            self.pair_table = get(self.pair.name).to(device=device, dtype=dtype).contiguous()
         if spec.streams:
             self._ones = torch.ones(spec.streams, dtype=torch.float32, device=device)
         # whoever runs the model works on a stream of their own: everything that loading enqueued (copies, re-laying of
@@ -131,10 +152,19 @@ class DecoderModel:
         before the last sum.  ``caches[i]`` is the cache view of run-order entry i (its own or the one
         it reads)."""
         n = ctx.n_tokens
+        ctx.shared = {key: ctx.arena.take((n, cols), self.dtype) for key, cols in self.step_buffers.items()}
         if self.spec.streams:
             # copies of the stream in 32-bit, all equal to the embedding's output; blocks update them in place
             resid = ctx.arena.take((n, self.spec.streams, self.spec.hidden), torch.float32)
-            ops.embed_streams(self.embed, ctx.token_ids, resid, scale=self.spec.embed_scale)
+            if self.pair is not None:
+                state = (getattr(ctx, "model_state", None) or {}).get(self.LAST_TOKEN)
+                if state is None:
+                    raise ValueError("the step's context holds no state for the tokens before its first ones (ctx.model_state)")
+                ops.embed_pair_streams(self.embed, self.pair_table, ctx.token_ids, ctx.positions, ctx.token_req, ctx.qo_indptr,
+                                       ctx.state_slots, state, resid, self.spec.embed_scale, self.pair.buckets, self.pair.mul_prev,
+                                       self.pair.mul_cur)
+            else:
+                ops.embed_streams(self.embed, ctx.token_ids, resid, scale=self.spec.embed_scale)
             # a block leaves its last sublayer's output unwritten (``ops.PendingWrite``): the next read writes it in passing
             pending = None
             carry = ctx.arena.take((n, self.spec.hidden), self.dtype)

@@ -34,6 +34,20 @@ def inverse_frequencies(rotary_dim: int, theta: float, scaling) -> torch.Tensor:
     return torch.where(between, (1 - t) * scaled / factor + t * scaled, scaled)
 
 
+def yarn_frequencies(rotary_dim: int, theta: float, yarn) -> tuple[torch.Tensor, float]:
+    """-> (float32 [rotary_dim / 2], factor on cosine and sine) for yarn = (factor, original, fast, slow): pairs whose
+    wavelength is long against ``original`` turn ``factor`` times slower, short ones as they are, a linear ramp between
+    (see ``config.spec.RopeSpec``).  Formed in 64-bit, then rounded once."""
+    factor, original, fast, slow = (float(v) for v in yarn)
+    j = torch.arange(rotary_dim // 2, dtype=torch.float64)
+    f = theta ** (-2.0 * j / rotary_dim)
+    at = lambda t: rotary_dim * math.log(original / (2 * math.pi * t)) / (2 * math.log(theta))
+    lo = max(math.floor(at(fast)), 0)
+    hi = min(math.ceil(at(slow)), rotary_dim - 1)
+    ramp = ((j - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+    return (f / factor * ramp + f * (1.0 - ramp)).to(torch.float32), 0.1 * math.log(factor) + 1.0
+
+
 class Rope:
     graph_safe = True
 
@@ -45,12 +59,21 @@ class Rope:
         self.max_positions = spec.max_positions
         self.interleaved, self.factor = bool(spec.interleaved), float(spec.cos_sin_factor)
         self.inv_freq: torch.Tensor | None = None
+        yarn = getattr(spec, "yarn", None)
+        if yarn is not None:
+            if spec.scaling is not None:
+                raise ValueError("a rotation has one frequency scaling, not two")
+            self._yarn_freq, mult = yarn_frequencies(spec.rotary_dim, spec.theta, yarn)
+            self.factor *= mult
 
     def wanted(self) -> dict:
         return {}
 
     def load(self, get, dtype, device) -> None:
-        self.inv_freq = inverse_frequencies(self.spec.rotary_dim, self.spec.theta, self.spec.scaling).to(device)
+        if getattr(self.spec, "yarn", None) is not None:
+            self.inv_freq = self._yarn_freq.to(device)
+        else:
+            self.inv_freq = inverse_frequencies(self.spec.rotary_dim, self.spec.theta, self.spec.scaling).to(device)
 
 
 class NoPosition:

@@ -1,8 +1,8 @@
 """Seeded random weights for any model spec, and a writer of whole model folders.
 
 The law of a tensor is what its part says in ``wanted()``: name -> (shape, role).  A role is a name in ``LAWS``
-(linear matrices and embedding tables are N(0, 0.02); norm weights are 1 + N(0, 0.02); "zeros" and "ones" for
-biases and gains that start neutral), or a function ``(shape, generator) -> float32 tensor`` on the generator's
+(linear matrices, embedding tables and biases are N(0, 0.02); norm weights are 1 + N(0, 0.02), or N(0, 0.1) for norms
+whose factor is one plus the stored weight ("around_zero"); "zeros" and "ones" for gains that start neutral), or a function ``(shape, generator) -> float32 tensor`` on the generator's
 device, for a part whose tensors want a law of their own (a decay, a convolution).
 Tensors are drawn in the sorted order of their names from one ``torch.Generator`` seeded with
 ``seed``, in 32-bit, then cast, so that a folder written here and the tensors made in memory from
@@ -17,7 +17,8 @@ from pathlib import Path
 import torch
 
 STD = 0.02
-LAWS = {"linear": (0.0, STD), "embedding": (0.0, STD), "norm": (1.0, STD), "zeros": (0.0, 0.0), "ones": (1.0, 0.0)}  # role -> (mean, std)
+LAWS = {"linear": (0.0, STD), "embedding": (0.0, STD), "norm": (1.0, STD), "zeros": (0.0, 0.0), "ones": (1.0, 0.0),
+        "bias": (0.0, STD), "around_zero": (0.0, 0.1)}  # role -> (mean, std)
 
 
 def draw(shape, role, gen: torch.Generator, dtype=torch.float32, draw_dtype=torch.float32) -> torch.Tensor:
