@@ -229,8 +229,33 @@ def vuzelix_config(shape: dict, layers: int | None = None):
     return replace(cfg, decay_rank=64, gate_rank=64)
 
 
+# Sizes for ``--design fetitar``: the Fetitar design at the widths, depths and head counts of the Llama shapes above.  Every
+# second layer is a latent-attention layer (the shape's heads with head_dim unrotated and head_dim / 2 rotated channels,
+# values of head_dim, a query latent of 3/8 of the width and a key/value latent of 512, YaRN-scaled rotation), the others
+# attention layers of the shape's heads and key/value heads with biases, whole-projection norms, distance slopes and mixed
+# values; windows of 1,024 positions; gated feed-forwards of the shape's inner size with biases; a pair table of 65,536 rows.
+def fetitar_config(shape: dict, layers: int | None = None):
+    from nanospec_amd.config import FetitarConfig
+
+    n = layers or shape["num_hidden_layers"]
+    heads, kvh, hd, ff, width = (shape["num_attention_heads"], shape["num_key_value_heads"], shape["head_dim"], shape["intermediate_size"],
+                                 shape["hidden_size"])
+    entries = []
+    for i in range(n):
+        mlp = {"kind": "dense", "ff": ff}
+        if i % 2 == 0:
+            m = dict(heads=heads, dim=hd, rot_dim=hd // 2, vdim=hd, q_rank=3 * width // 8, kv_rank=512, scale=(hd + hd // 2) ** -0.5,
+                     mask={"size": 1024}, rot={"base": 1e6, "dims": hd // 2, "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}})
+            entries.append({"type": "latent_attention", "mixer": m, "mlp": mlp})
+        else:
+            m = dict(heads=heads, kv_heads=kvh, dim=hd, vdim=hd, scale=hd ** -0.5, mask={"size": 1024}, v_mix=True)
+            entries.append({"type": "attention", "mixer": m, "mlp": mlp})
+    return FetitarConfig.from_hf({"architecture": "Fetitar", "vocab": shape["vocab_size"], "width": width, "norm": {"eps": 1e-6},
+                                  "embedding": {"scale": 1.0, "bigram": {"buckets": 65536, "mul_prev": 127, "mul_cur": 7}}, "layers": entries})
+
+
 def design_compare(a) -> int:
-    """``--design vuzelix``: prefill and decode throughput of the Vuzelix design beside the Llama model of the same shape,
+    """``--design NAME``: prefill and decode throughput of that design beside the Llama model of the same shape,
     one JSON line.  The default workload and its output are not touched by this option."""
     import types
 
@@ -245,10 +270,11 @@ def design_compare(a) -> int:
     dtype = torch.bfloat16 if a.dtype == "bf16" else torch.float32
     llama = LlamaConfig.from_hf(dict(model_type="llama", **{k: v for k, v in shape.items() if k != "rope_scaling"},
                                      rope_scaling=dict(rope_type="llama3", **shape["rope_scaling"])))
-    vz = vuzelix_config(shape)
+    design = a.design
+    vz = vuzelix_config(shape) if design == "vuzelix" else fetitar_config(shape)
     out = {}
     k = min(a.steps, 128)
-    for name, cfg in (("llama", llama), ("vuzelix", vz)):
+    for name, cfg in (("llama", llama), (design, vz)):
         model = random_model(cfg, seed=0, dtype=dtype, on_device=True)
         facts = types.SimpleNamespace(vocab_size=shape["vocab_size"])
         row = {}
@@ -262,13 +288,13 @@ def design_compare(a) -> int:
         out[name] = row
         del model
         torch.cuda.empty_cache()
-    ratio = {key: round(out["vuzelix"][key] / out["llama"][key], 3) for key in out["llama"] if key.endswith("tok_s")}
-    print(json.dumps({"metric": f"prefill and decode tok/s of the Vuzelix design beside Llama at the {SHAPE_NAMES[a.shape]} ({a.dtype})",
+    ratio = {key: round(out[design][key] / out["llama"][key], 3) for key in out["llama"] if key.endswith("tok_s")}
+    layers = [l.type + ("*" if getattr(l, "kv_from", None) is not None else "") for l in vz.layers]
+    print(json.dumps({"metric": f"prefill and decode tok/s of the {design.capitalize()} design beside Llama at the {SHAPE_NAMES[a.shape]} ({a.dtype})",
                       "unit": "tok/s", "n_gpus": 1, "dtype": a.dtype, "data": "synthetic: random weights, uniform random token ids",
                       "config": {"shape": SHAPE_NAMES[a.shape], "layers": shape["num_hidden_layers"], "hidden": shape["hidden_size"],
-                                 "vuzelix_layers": [l.type + ("*" if l.kv_from is not None else "") for l in vz.layers], "streams": vz.streams,
-                                 "page_size": 16, "decode_steps": k},
-                      "llama": out["llama"], "vuzelix": out["vuzelix"], "vuzelix_over_llama": ratio}), flush=True)
+                                 f"{design}_layers": layers, "streams": getattr(vz, "streams", 1), "page_size": 16, "decode_steps": k},
+                      "llama": out["llama"], design: out[design], f"{design}_over_llama": ratio}), flush=True)
     return 0
 
 
@@ -288,7 +314,7 @@ def main() -> int:
                     help="instead of the benchmark: continuous batching of this many requests (prompts of 16 to 1,024 tokens, 128 new "
                          "tokens each, prompts in portions of 512)")
     ap.add_argument("--shape", default="8b", choices=sorted(SHAPES), help="the benchmark's shape is 8b; the others are for profiles")
-    ap.add_argument("--design", default=None, choices=["vuzelix"],
+    ap.add_argument("--design", default=None, choices=["vuzelix", "fetitar"],
                     help="instead of the benchmark: prefill and decode of this design beside the Llama model of the same --shape")
     a = ap.parse_args()
     if a.gpus != 1:
