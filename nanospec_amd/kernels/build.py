@@ -30,6 +30,7 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
 
 CORE_SOURCES = ["elementwise.hip", "gemm_generic.hip", "attn_generic.hip", "sampling.hip", "gemm_bf16.hip", "gemm_wide.hip", "graph.hip", "streams.hip", "delta.hip", "latent.hip"]
 ATTN_SOURCES = ["attn_mfma.hip"]
+WIDE_SOURCES = ["attn_wide.hip"]
 
 _loaded: dict[str, ctypes.CDLL] = {}
 
@@ -134,12 +135,28 @@ def attn(head_dim: int, page_size: int) -> ctypes.CDLL:
     return load_library(attn_name(head_dim, page_size), ATTN_SOURCES, _attn_defines(head_dim, page_size))
 
 
-def build_all(attn_variants=((16, 4), (32, 8), (64, 16), (128, 16)), force: bool = True, jobs: int | None = None) -> None:
-    """Compile the core library and the attention library of each given (head size, page size), ``jobs`` compilers at a
-    time (by default one per processor, at most eight)."""
+def wide_name(head_dim: int, value_dim: int, page_size: int) -> str:
+    return f"ns_wide_hd{head_dim}_v{value_dim}_p{page_size}"
+
+
+def _wide_defines(head_dim: int, value_dim: int, page_size: int) -> list[str]:
+    return [f"-DNS_HEAD_DIM={head_dim}", f"-DNS_VALUE_DIM={value_dim}", f"-DNS_PAGE_SIZE={page_size}"]
+
+
+def attn_wide(head_dim: int, value_dim: int, page_size: int) -> ctypes.CDLL:
+    """The matrix-core attention kernel for keys and values of two sizes (and wide heads), one library per (key size, value
+    size, page size), compiled on first use."""
+    return load_library(wide_name(head_dim, value_dim, page_size), WIDE_SOURCES, _wide_defines(head_dim, value_dim, page_size))
+
+
+def build_all(attn_variants=((16, 4), (32, 8), (64, 16), (128, 16)), force: bool = True, jobs: int | None = None, wide_variants=()) -> None:
+    """Compile the core library, the attention library of each given (head size, page size) and the two-size attention
+    library of each given (key size, value size, page size), ``jobs`` compilers at a time (by default one per processor, at
+    most eight)."""
     from concurrent.futures import ThreadPoolExecutor
 
     work = [("ns_core", CORE_SOURCES, [])] + [(attn_name(hd, page), ATTN_SOURCES, _attn_defines(hd, page)) for hd, page in attn_variants]
+    work += [(wide_name(hd, vd, page), WIDE_SOURCES, _wide_defines(hd, vd, page)) for hd, vd, page in wide_variants]
     jobs = jobs or max(1, min(8, os.cpu_count() or 1))
     with ThreadPoolExecutor(max_workers=jobs) as pool:
         for done in [pool.submit(compile_library, name, sources, defines, force) for name, sources, defines in work]:

@@ -762,6 +762,45 @@ def attention_mfma(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_
     return out
 
 
+def wide_attention_takes(dtype, head_dim: int, v_dim: int, page_size: int) -> bool:
+    return (dtype == torch.bfloat16 and head_dim % 16 == 0 and 16 <= head_dim <= 1024 and v_dim % 16 == 0 and 16 <= v_dim <= 512
+            and page_size >= 4 and page_size & (page_size - 1) == 0)
+
+
+def attention_wide(q, out, k_cache, v_cache, tiles, block_table, heads: int, kv_heads: int, head_dim: int, v_dim: int, scale: float,
+                   window: int = 0, hp: int = 1, splits: int = 1, workspace: tuple[torch.Tensor, torch.Tensor] | None = None, qt: int = 1,
+                   slope_exp: float = 0.0) -> torch.Tensor:
+    """bfloat16 attention on the matrix cores for keys of ``head_dim`` and values of ``v_dim`` channels (multiples of 16 up
+    to 1,024 and 512), over the tiles of ``tiles`` (as for ``attention_mfma``): ``hp`` heads of a group times 16/hp tokens
+    are one wave's columns, ``qt`` such sets of tokens a tile.  ``splits`` > 1 cuts every tile's keys into ranges and needs
+    ``workspace`` = (part_o, part_ml) float32 tensors.  ``slope_exp``: as for ``attention_generic``."""
+    page = _check_attn(q, out, k_cache, v_cache, heads, kv_heads, head_dim, v_dim)
+    if not wide_attention_takes(q.dtype, head_dim, v_dim, page):
+        raise KernelRefused(f"attention_wide takes bfloat16, key sizes that are multiples of 16 up to 1024, value sizes up to 512 and page "
+                            f"sizes that are powers of two from 4; got {q.dtype}, sizes {head_dim} and {v_dim}, page {page}")
+    _gpu(tiles, block_table)
+    _i32(tiles, "tiles"), _i32(block_table, "block_table")
+    if tiles.dim() != 2 or tiles.shape[1] != TILE_INTS or tiles.data_ptr() % 16:
+        raise KernelRefused(f"attention_wide: tiles must be int32 [n_tiles, {TILE_INTS}], 16-byte aligned")
+    if hp not in (1, 2, 4, 8, 16) or not 1 <= qt <= 4:
+        raise KernelRefused("attention_wide: hp is a power of two up to 16, qt 1 to 4")
+    n_tiles = tiles.shape[0]
+    po = pm = None
+    if splits > 1:
+        if workspace is None or splits > 64:
+            raise KernelRefused("attention_wide: 2 to 64 key ranges are taken, with a workspace")
+        po, pm = workspace
+        cols = n_tiles * (qt * 16 // hp) * heads
+        if po.dtype != torch.float32 or pm.dtype != torch.float32 or po.numel() < cols * splits * v_dim or pm.numel() < cols * splits * 2:
+            raise KernelRefused("attention_wide: workspace too small")
+    lib = build.attn_wide(head_dim, v_dim, page)
+    _check(lib.ns_attn_wide(_ptr(out), _ptr(po), _ptr(pm), _ptr(q), c_int(q.stride(0)), _ptr(k_cache), _ptr(v_cache), _ptr(tiles),
+                            _ptr(block_table), c_int(block_table.stride(0)), c_int(n_tiles), c_int(heads), c_int(kv_heads), c_int(page),
+                            c_int(hp), c_int(splits), c_int(window), c_float(scale), c_int(qt), c_float(slope_exp), _stream()),
+           "attention_wide")
+    return out
+
+
 def attention_prompt_form(head_dim: int, page_size: int) -> int:
     """Which kernel of the library for this head and page size takes prompt portions in tiles of 32 tokens: 32 the one
     on the 32x32 matrix instruction with loads straight into LDS, 16 the one on the 16x16 instruction with keys shared

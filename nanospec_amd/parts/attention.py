@@ -134,6 +134,45 @@ def launch_plans(ctx, group: int, kv_heads: int, head_dim: int, span: int = 0) -
     return plans
 
 
+WIDE_RANGE_KEYS = 128  # the fewest keys that a range of a row's keys is worth a wave of its own in the two-size kernel
+
+
+def wide_attention(ctx, q, out, cache, table, heads: int, kv_heads: int, head_dim: int, v_dim: int, scale: float, window: int = 0,
+                   slope_exp: float = 0.0):
+    """Launch ``ops.attention_wide`` (keys and values of two sizes on the matrix cores) over the tile lists of the batch:
+    prompt portions as sets of 16 tokens of one head, decode rows with up to 16 heads of a group in one wave's columns and
+    the keys cut into ranges until the launch fills the GPU (an item of that kernel is one wave)."""
+    units = ops.compute_units(ctx.token_ids.device)
+    group = heads // kv_heads
+    chunk_tiles, decode_tiles = TilePlan.views(ctx)
+    take = ctx.arena.take
+    if chunk_tiles.shape[0]:
+        qt = TilePlan.TOKENS // 16
+        waves = chunk_tiles.shape[0] * qt * heads
+        longest = min(ctx.max_chunk_kv, window + TilePlan.TOKENS) if window else ctx.max_chunk_kv
+        splits = max(1, min(16, 4 * units // max(1, waves), longest // (4 * WIDE_RANGE_KEYS)))
+        ws = None
+        if splits > 1:
+            cols = chunk_tiles.shape[0] * TilePlan.TOKENS * heads
+            ws = (take((cols * splits * v_dim,), torch.float32), take((cols * splits * 2,), torch.float32))
+        ops.attention_wide(q, out, cache.k, cache.v, chunk_tiles, table, heads, kv_heads, head_dim, v_dim, scale, window=window, hp=1,
+                           splits=splits, workspace=ws, qt=qt, slope_exp=slope_exp)
+    if decode_tiles.shape[0]:
+        hp = 1
+        while hp < min(group, 16):
+            hp *= 2
+        waves = decode_tiles.shape[0] * kv_heads * -(-group // hp)
+        longest = min(ctx.max_kv_len, window) if window else ctx.max_kv_len
+        splits = max(1, min(32, 4 * units // max(1, waves), -(-longest // WIDE_RANGE_KEYS)))
+        ws = None
+        if splits > 1:
+            cols = decode_tiles.shape[0] * (16 // hp) * heads
+            ws = (take((cols * splits * v_dim,), torch.float32), take((cols * splits * 2,), torch.float32))
+        ops.attention_wide(q, out, cache.k, cache.v, decode_tiles, table, heads, kv_heads, head_dim, v_dim, scale, window=window, hp=hp,
+                           splits=splits, workspace=ws, qt=1, slope_exp=slope_exp)
+    return out
+
+
 class Attention:
     graph_safe = True
     ends_in_residual = True  # forward takes residual=IntoResidual
@@ -328,6 +367,10 @@ class Attention:
                 ops.attention_mfma(qkv, att, cache.k, cache.v, plan.tiles, table, s.heads, s.kv_heads, s.head_dim, s.softmax_scale,
                                    window=s.window, hp=plan.hp, splits=plan.splits, workspace=plan.workspace, qt=plan.qt, coop=plan.coop,
                                    chunk=s.chunk, cap=s.score_cap, sink=s.sink)
+        elif not (s.chunk or s.score_cap or s.sink) and ops.wide_attention_takes(x.dtype, s.head_dim, s.v_dim, cache.k.shape[2]):
+            # bfloat16, values of another size than the keys or a bias by distance: the two-size matrix-core kernel
+            wide_attention(ctx, qkv, att, cache, table, s.heads, s.kv_heads, s.head_dim, s.v_dim, s.softmax_scale, window=s.window,
+                           slope_exp=s.slope_exp)
         else:
             ops.attention_generic(qkv, att, cache.k, cache.v, ctx.token_req, ctx.positions, table, s.heads, s.kv_heads, s.head_dim,
                                   s.softmax_scale, window=s.window, v_dim=s.v_dim, chunk=s.chunk, cap=s.score_cap, sink=s.sink,

@@ -20,7 +20,7 @@ import torch
 
 from ..kernels import ops
 from . import registry
-from .attention import TILES, launch_plans
+from .attention import TILES, wide_attention
 from .linear import LinearWeight
 from .needs import PagedNeed
 
@@ -98,8 +98,11 @@ class LatentAttention:
         q = self.uq(cq, out=take((n, H * (D + R)), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)
         q_lat = ops.latent_q_absorb(q, self.uk, pos.inv_freq, self._factor, ctx.positions, H, D, R, C, out=take((n, H * (C + R)), x.dtype))
         o_lat = take((n, H * C), x.dtype)
-        ops.attention_generic(q_lat, o_lat, cache.k, cache.v, ctx.token_req, ctx.positions, table, H, 1, C + R, s.softmax_scale,
-                              window=s.window, v_dim=C)
+        if ops.wide_attention_takes(x.dtype, C + R, C, cache.k.shape[2]):
+            wide_attention(ctx, q_lat, o_lat, cache, table, H, 1, C + R, C, s.softmax_scale, window=s.window)
+        else:
+            ops.attention_generic(q_lat, o_lat, cache.k, cache.v, ctx.token_req, ctx.positions, table, H, 1, C + R, s.softmax_scale,
+                                  window=s.window, v_dim=C)
         att = ops.latent_out(o_lat, self.uv_t, gate, H, C, E, out=take((n, H * E), x.dtype))
         return self.wo(att, out=out if out is not None else take((n, s.hidden), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)
 

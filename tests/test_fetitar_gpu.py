@@ -669,3 +669,55 @@ def test_gated_feed_forward_with_biases(dtype, rows):
     # with the last bias left to the caller
     got = part.forward(Ctx, x.to(DEV), add_out_bias=False).cpu().double() + w["f.down.b"].double()
     assert (got - ref).abs().max() / ref.abs().max() <= (2e-5 if dtype == torch.float32 else 0.03)
+
+
+@pytest.mark.parametrize("HD,VD,page,H,G,window,slope", [(48, 32, 4, 4, 2, 37, 8.0), (96, 64, 16, 4, 1, 0, 8.0), (80, 48, 8, 3, 3, 20, 0.0),
+                                                         (160, 128, 16, 24, 1, 100, 0.0), (288, 176, 16, 2, 1, 70, 2.0)])
+def test_two_size_matrix_core_attention(HD, VD, page, H, G, window, slope):
+    """Keys and values of two sizes on the matrix cores: a prompt portion behind cached keys beside three single tokens of
+    other requests, with the keys in one range and cut into ranges; against the plain rows."""
+    from nanospec_amd.cache.storage import PagedView
+    from nanospec_amd.kernels import ops
+    from nanospec_amd.parts.attention import TilePlan
+
+    g = torch.Generator().manual_seed(HD + VD)
+    lens, starts = [45, 1, 1, 1], [150, 0, 299, 64]
+    total = [s + n for s, n in zip(starts, lens)]
+    pages_of = [-(-t // page) for t in total]
+    ids = list(range(sum(pages_of)))
+    random.Random(3).shuffle(ids)
+    tables, at = [], 0
+    for n in pages_of:
+        tables.append(ids[at : at + n])
+        at += n
+    ks = [torch.randn(t, G, HD, generator=g).to(torch.bfloat16) for t in total]
+    vs = [torch.randn(t, G, VD, generator=g).to(torch.bfloat16) for t in total]
+    kc, vc = torch.zeros(len(ids), G, page, HD, dtype=torch.bfloat16), torch.zeros(len(ids), G, VD, page, dtype=torch.bfloat16)
+    for b, tab in enumerate(tables):
+        for t in range(total[b]):
+            kc[tab[t // page], :, t % page] = ks[b][t]
+            vc[tab[t // page], :, :, t % page] = vs[b][t]
+    kc, vc = kc.to(DEV), vc.to(DEV)
+    q = torch.randn(sum(lens), H, HD, generator=g).to(torch.bfloat16)
+    ctx = step_context(lens, starts, tables)
+    scale = 0.5 / math.sqrt(HD)
+    refs, row = [], 0
+    for b, n in enumerate(lens):
+        positions = list(range(starts[b], starts[b] + n))
+        refs.append(plain_rows(q[row : row + n].double(), ks[b].double(), vs[b].double(), scale, window,
+                               torch.tensor([2.0 ** (-slope * (h + 1) / H) for h in range(H)], dtype=F) if slope else None, positions))
+        row += n
+    ref = torch.cat(refs).reshape(sum(lens), H * VD)
+    chunk_tiles, decode_tiles = TilePlan.views(ctx)
+    hp = 1
+    while hp < min(H // G, 16):
+        hp *= 2
+    for splits in (1, 3):
+        out = torch.zeros(sum(lens), H * VD, dtype=torch.bfloat16, device=DEV)
+        for tiles, kw in ((chunk_tiles, dict(hp=1, qt=2)), (decode_tiles, dict(hp=hp, qt=1))):
+            cols = tiles.shape[0] * (kw["qt"] * 16 // kw["hp"]) * H
+            ws = (torch.zeros(cols * splits * VD, device=DEV), torch.zeros(cols * splits * 2, device=DEV)) if splits > 1 else None
+            ops.attention_wide(q.reshape(sum(lens), H * HD).to(DEV), out, kc, vc, tiles, ctx.block_tables[0], H, G, HD, VD, scale, window=window,
+                               splits=splits, workspace=ws, slope_exp=slope, **kw)
+        err = (out.cpu().double() - ref).abs().max() / ref.abs().max()
+        assert err <= 0.02, (splits, err)
