@@ -29,7 +29,7 @@ constexpr int DT = VD / 16;                   // 16-channel tiles of the output
 constexpr bool WIDE = HD % 32 == 0;           // q.k with the k=32 instruction, else with k=16
 constexpr int NQ = WIDE ? HD / 32 : HD / 16;  // q.k instructions per 16-key tile
 constexpr int TILE_INTS = 8;
-constexpr int VPIECE = DT < 8 ? DT : 8;       // channel tiles of the values that are asked for together
+constexpr int VPIECE = DT < 16 ? DT : 16;       // channel tiles of the values that are asked for together
 
 typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
 typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 bf16x4;

@@ -8,6 +8,7 @@
 //                    c into the V page, sigmoid of the gate logits (32-bit)
 //   latent_q_absorb  q [H][D + R] -> [H][C + R]: the unrotated part through Uk_h^T, the rotated part turned by its position
 //   latent_out       o [H][C] -> [H][E] through Uv_h, times the gate
+//   headwise_mfma    the two per-head products on the matrix cores (bfloat16, sizes that are multiples of 32 and 16)
 // Norms, angles, rotations, the sigmoid and every sum are 32-bit.  Rotation pairs channel i with i + R/2.
 #include "common.h"
 #include "rope.h"
@@ -74,7 +75,7 @@ template <typename T>
 __global__ __launch_bounds__(256) void latent_q_absorb_kernel(const T* __restrict__ q, int q_stride, const T* __restrict__ uk,
                                                               const float* __restrict__ inv_freq, float factor,
                                                               const int* __restrict__ positions, T* __restrict__ out, int n, int H, int D,
-                                                              int R, int C) {
+                                                              int R, int C, int absorb) {
   extern __shared__ float q_s[];  // [LAT_TOKENS][D]
   const int t0 = blockIdx.x * LAT_TOKENS, h = blockIdx.y;
   const int nt = min(LAT_TOKENS, n - t0);
@@ -84,7 +85,7 @@ __global__ __launch_bounds__(256) void latent_q_absorb_kernel(const T* __restric
   }
   __syncthreads();
   const T* w = uk + (size_t)h * D * C;
-  for (int c = threadIdx.x; c < C; c += blockDim.x) {
+  for (int c = threadIdx.x; c < (absorb ? C : 0); c += blockDim.x) {
     float acc[LAT_TOKENS] = {};
     for (int d = 0; d < D; ++d) {
       const float wv = to_f(w[(size_t)d * C + c]);
@@ -109,17 +110,18 @@ __global__ __launch_bounds__(256) void latent_q_absorb_kernel(const T* __restric
 }
 
 extern "C" int ns_latent_q_absorb(const void* q, int q_stride, const void* uk, const float* inv_freq, float factor, const int* positions,
-                                  void* out, int n, int H, int D, int R, int C, int dtype, hipStream_t stream) {
+                                  void* out, int n, int H, int D, int R, int C, int absorb, int dtype, hipStream_t stream) {
   if (n <= 0 || H <= 0 || H > 65535 || D <= 0 || R < 0 || R % 2 || C <= 0 || (size_t)LAT_TOKENS * D * sizeof(float) > 64 * 1024) return NS_ERR_BAD_ARG;
+  if (!absorb && !uk) uk = q;  // (not read)
   const dim3 grid((n + LAT_TOKENS - 1) / LAT_TOKENS, H);
   const size_t smem = (size_t)LAT_TOKENS * D * sizeof(float);
   const int threads = C >= 256 ? 256 : (C >= 128 ? 128 : 64);
   if (dtype == NS_DTYPE_F32)
     latent_q_absorb_kernel<float><<<grid, threads, smem, stream>>>((const float*)q, q_stride, (const float*)uk, inv_freq, factor, positions,
-                                                                   (float*)out, n, H, D, R, C);
+                                                                   (float*)out, n, H, D, R, C, absorb);
   else if (dtype == NS_DTYPE_BF16)
     latent_q_absorb_kernel<bf16_t><<<grid, threads, smem, stream>>>((const bf16_t*)q, q_stride, (const bf16_t*)uk, inv_freq, factor, positions,
-                                                                    (bf16_t*)out, n, H, D, R, C);
+                                                                    (bf16_t*)out, n, H, D, R, C, absorb);
   else
     return NS_ERR_UNSUPPORTED;
   return ns_launch_status();
@@ -164,5 +166,73 @@ extern "C" int ns_latent_out(const void* o, const void* uv_t, const float* gate,
     latent_out_kernel<bf16_t><<<grid, threads, smem, stream>>>((const bf16_t*)o, (const bf16_t*)uv_t, gate, (bf16_t*)out, n, H, C, E);
   else
     return NS_ERR_UNSUPPORTED;
+  return ns_launch_status();
+}
+
+// ------------------------------------------------------------------------------------------------
+// The two per-head products on the matrix cores (bfloat16): out[t][h][n] = gate[t][h] * sum_k x[t][h][k] w[h][n][k], with
+// w [H][N][K] (every head's matrix as [out, in] rows), K a multiple of 32 and N of 16.  Kept transposed, D[n][token] =
+// W[n][:] . X[token][:], so that both operands are 16-byte loads of consecutive k straight from memory and a lane ends up
+// with four consecutive n of one token.  A wave takes 16 tokens of one head and NT tiles of 16 outputs; x is re-read per
+// wave from the caches (16 tokens of one head are a few KB).
+// ------------------------------------------------------------------------------------------------
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 hw_bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(__bf16)))) __bf16 hw_bf16x4;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float hw_f32x4;
+
+template <int NT>
+__global__ __launch_bounds__(256) void headwise_mfma_kernel(const bf16_t* __restrict__ x, long x_row, int x_head, const bf16_t* __restrict__ w,
+                                                            const float* __restrict__ gate, bf16_t* __restrict__ out, long out_row,
+                                                            int out_head, int n_tokens, int H, int N, int K) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int t0 = blockIdx.x * 16, h = blockIdx.y;
+  const int n0 = (blockIdx.z * 4 + wave) * NT * 16;
+  if (n0 >= N) return;
+  const int token = t0 + c;
+  const bool tok_ok = token < n_tokens;
+  const bf16_t* xp = x + (size_t)(tok_ok ? token : 0) * x_row + (size_t)h * x_head + g * 8;
+  const bf16_t* wp[NT];
+#pragma unroll
+  for (int i = 0; i < NT; ++i) wp[i] = w + ((size_t)h * N + min(n0 + i * 16 + c, N - 1)) * K + g * 8;
+  hw_f32x4 acc[NT];
+#pragma unroll
+  for (int i = 0; i < NT; ++i) acc[i] = hw_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    hw_bf16x8 b = *reinterpret_cast<const hw_bf16x8*>(xp + k0);
+    if (!tok_ok) b = hw_bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+    hw_bf16x8 a[NT];
+#pragma unroll
+    for (int i = 0; i < NT; ++i) a[i] = *reinterpret_cast<const hw_bf16x8*>(wp[i] + k0);
+#pragma unroll
+    for (int i = 0; i < NT; ++i) acc[i] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b, acc[i], 0, 0, 0);
+  }
+  if (!tok_ok) return;
+  const float gt = gate ? gate[(size_t)token * H + h] : 1.f;
+#pragma unroll
+  for (int i = 0; i < NT; ++i) {
+    const int n = n0 + i * 16 + g * 4;  // acc[i][j] is output n + j of this lane's token
+    if (n < N) {
+      const hw_bf16x4 r = {(bf16_t)(acc[i][0] * gt), (bf16_t)(acc[i][1] * gt), (bf16_t)(acc[i][2] * gt), (bf16_t)(acc[i][3] * gt)};
+      *reinterpret_cast<hw_bf16x4*>(out + (size_t)token * out_row + (size_t)h * out_head + n) = r;
+    }
+  }
+}
+
+extern "C" int ns_headwise_bf16(const void* x, long x_row, int x_head, const void* w, const float* gate, void* out, long out_row, int out_head,
+                                int n_tokens, int H, int N, int K, hipStream_t stream) {
+  if (n_tokens <= 0 || H <= 0 || H > 65535 || N <= 0 || N % 16 || K <= 0 || K % 32 || (x_row & 7) || (x_head & 7) || (out_row & 3) || (out_head & 3) ||
+      ((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)out & 7))
+    return NS_ERR_BAD_ARG;
+  const int tiles = N / 16;
+  if (tiles >= 16) {
+    const dim3 grid((n_tokens + 15) / 16, H, (tiles + 15) / 16);
+    headwise_mfma_kernel<4><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, gate, (bf16_t*)out, out_row, out_head,
+                                                      n_tokens, H, N, K);
+  } else {
+    const dim3 grid((n_tokens + 15) / 16, H, (tiles + 3) / 4);
+    headwise_mfma_kernel<1><<<grid, 256, 0, stream>>>((const bf16_t*)x, x_row, x_head, (const bf16_t*)w, gate, (bf16_t*)out, out_row, out_head,
+                                                      n_tokens, H, N, K);
+  }
   return ns_launch_status();
 }

@@ -1070,20 +1070,48 @@ def latent_prep(proj: torch.Tensor, q_norm: torch.Tensor, c_norm: torch.Tensor, 
                                        c_int(page), c_float(eps), c_int(_dtype_code(proj)), _stream()), "latent_prep")
 
 
-def latent_q_absorb(q: torch.Tensor, uk: torch.Tensor, inv_freq: torch.Tensor, factor: float, positions, heads: int, dim: int, rot: int,
+def headwise_takes(dtype, n_out: int, k: int, x_head: int, out_head: int) -> bool:
+    """Whether ``headwise_product`` takes these sizes: bfloat16, K a multiple of 32, N of 16, heads 16 and 8 bytes apart."""
+    return dtype == torch.bfloat16 and k % 32 == 0 and n_out % 16 == 0 and x_head % 8 == 0 and out_head % 4 == 0
+
+
+def headwise_product(x: torch.Tensor, x_head: int, w: torch.Tensor, out: torch.Tensor, out_head: int, gate: torch.Tensor | None = None) -> torch.Tensor:
+    """One product per head on the matrix cores: out[t, h * out_head + n] = gate[t, h] * sum_k x[t, h * x_head + k] w[h, n, k]
+    for w [heads, N, K] (bfloat16).  A head's part of a row of ``x`` may be wider than K and of ``out`` wider than N: the
+    rest is not read and not written."""
+    _gpu(x, w, out, gate)
+    H, N, K = w.shape
+    n = x.shape[0]
+    if (x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16 or out.dtype != torch.bfloat16 or not w.is_contiguous() or x.dim() != 2 or out.dim() != 2
+            or x.stride(1) != 1 or out.stride(1) != 1 or out.shape[0] != n or x.shape[1] < (H - 1) * x_head + K or out.shape[1] < (H - 1) * out_head + N
+            or K > x_head or N > out_head or not headwise_takes(x.dtype, N, K, x_head, out_head) or x.stride(0) % 8 or out.stride(0) % 4):
+        raise KernelRefused("headwise_product: bfloat16 x [tokens, heads * x_head], w [heads, N, K] with K a multiple of 32 and N of 16")
+    if gate is not None and _f32(gate, "gate").shape != (n, H):
+        raise KernelRefused(f"headwise_product: gate is float32 [{n}, {H}]")
+    _check(build.core().ns_headwise_bf16(_ptr(x), ctypes.c_long(x.stride(0)), c_int(x_head), _ptr(w), _ptr(gate), _ptr(out),
+                                         ctypes.c_long(out.stride(0)), c_int(out_head), c_int(n), c_int(H), c_int(N), c_int(K), _stream()),
+           "headwise_product")
+    return out
+
+
+def latent_q_absorb(q: torch.Tensor, uk: torch.Tensor | None, inv_freq: torch.Tensor, factor: float, positions, heads: int, dim: int, rot: int,
                     latent: int, out: torch.Tensor) -> torch.Tensor:
     """q [tokens, heads * (dim + rot)] -> out [tokens, heads * (latent + rot)]: per head, the first ``dim`` values through
     that head's key matrix, out[c] = sum_d q[d] uk[head * dim + d, c] (``uk`` [heads * dim, latent]), and the ``rot`` values
-    behind them rotated by the position."""
+    behind them rotated by the position.  ``uk`` = None: the rotation alone (the product is the caller's)."""
     _gpu(q, uk, inv_freq, positions, out)
     n = positions.numel()
     _i32(positions, "positions"), _f32(inv_freq, "inv_freq")
+    absorb = uk is not None
+    if uk is None:
+        uk = torch.empty((heads * dim, latent), dtype=q.dtype, device="meta")
     if (q.dim() != 2 or q.shape != (n, heads * (dim + rot)) or q.stride(1) != 1 or uk.shape != (heads * dim, latent) or not uk.is_contiguous()
             or uk.dtype != q.dtype or out.shape != (n, heads * (latent + rot)) or not out.is_contiguous() or out.dtype != q.dtype or rot % 2
             or inv_freq.numel() < max(1, rot // 2) or dim > 2048):
         raise KernelRefused("latent_q_absorb: q [tokens, heads * (dim + rot)], uk [heads * dim, latent], out [tokens, heads * (latent + rot)]")
-    _check(build.core().ns_latent_q_absorb(_ptr(q), c_int(q.stride(0)), _ptr(uk), _ptr(inv_freq), c_float(factor), _ptr(positions), _ptr(out),
-                                           c_int(n), c_int(heads), c_int(dim), c_int(rot), c_int(latent), c_int(_dtype_code(q)), _stream()),
+    _check(build.core().ns_latent_q_absorb(_ptr(q), c_int(q.stride(0)), _ptr(uk if absorb else None), _ptr(inv_freq), c_float(factor),
+                                           _ptr(positions), _ptr(out), c_int(n), c_int(heads), c_int(dim), c_int(rot), c_int(latent),
+                                           c_int(1 if absorb else 0), c_int(_dtype_code(q)), _stream()),
            "latent_q_absorb")
     return out
 

@@ -134,7 +134,7 @@ def launch_plans(ctx, group: int, kv_heads: int, head_dim: int, span: int = 0) -
     return plans
 
 
-WIDE_RANGE_KEYS = 128  # the fewest keys that a range of a row's keys is worth a wave of its own in the two-size kernel
+WIDE_RANGE_KEYS = 64  # the fewest keys that a range of a row's keys is worth a wave of its own in the two-size kernel
 
 
 def wide_attention(ctx, q, out, cache, table, heads: int, kv_heads: int, head_dim: int, v_dim: int, scale: float, window: int = 0,

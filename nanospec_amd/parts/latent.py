@@ -64,8 +64,14 @@ class LatentAttention:
         self.first = LinearWeight(torch.cat([to(n["dq"]), to(n["dkv"])] + ([to(n["g"])] if s.gate else [])).contiguous(), keep_plain=plain)
         self.dq_norm, self.dkv_norm = to(n["dq_norm"]), to(n["dkv_norm"])
         self.uq = LinearWeight(to(n["uq"]), keep_plain=plain)
-        self.uk = to(n["uk"])  # [heads * dim, latent]: a head's rows are its Uk
-        self.uv_t = to(n["uv"]).view(s.heads, s.value_dim, s.kv_rank).transpose(1, 2).contiguous()  # [heads, latent, value]
+        # the two per-head matrices, each in the layout its kernel walks: on the matrix cores (bfloat16, sizes that fit) every
+        # head's matrix as [out, in] rows; otherwise as the plain kernels of ``csrc/latent.hip`` read them
+        D, R, E, C = s.head_dim, s.rot_dim, s.value_dim, s.kv_rank
+        self._mfma_q = ops.headwise_takes(dtype, C, D, D + R, C + R) and s.hidden % 8 == 0 and s.q_rank % 8 == 0
+        self._mfma_o = ops.headwise_takes(dtype, E, C, C, E)
+        uk, uv = to(n["uk"]), to(n["uv"])
+        self.uk = uk.view(s.heads, D, C).transpose(1, 2).contiguous() if self._mfma_q else uk  # [heads, latent, dim] | [heads * dim, latent]
+        self.uv = uv.view(s.heads, E, C) if self._mfma_o else uv.view(s.heads, E, C).transpose(1, 2).contiguous()  # [heads, value, latent] | [heads, latent, value]
         self.wo = LinearWeight(to(n["o"]), keep_plain=plain)
         self.position.load(get, dtype, device)
         self._factor = float(getattr(self.position, "factor", 1.0))
@@ -96,14 +102,21 @@ class LatentAttention:
         ops.latent_prep(proj, self.dq_norm, self.dkv_norm, pos.inv_freq, self._factor, ctx.positions, ctx.token_req, table, cache.k, cache.v,
                         s.q_rank, C, R, H if s.gate else 0, s.norm_eps, cq, gate)
         q = self.uq(cq, out=take((n, H * (D + R)), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)
-        q_lat = ops.latent_q_absorb(q, self.uk, pos.inv_freq, self._factor, ctx.positions, H, D, R, C, out=take((n, H * (C + R)), x.dtype))
+        q_lat = take((n, H * (C + R)), x.dtype)
+        if self._mfma_q:
+            ops.headwise_product(q, D + R, self.uk, q_lat, C + R)
+        ops.latent_q_absorb(q, None if self._mfma_q else self.uk, pos.inv_freq, self._factor, ctx.positions, H, D, R, C, out=q_lat)
         o_lat = take((n, H * C), x.dtype)
         if ops.wide_attention_takes(x.dtype, C + R, C, cache.k.shape[2]):
             wide_attention(ctx, q_lat, o_lat, cache, table, H, 1, C + R, C, s.softmax_scale, window=s.window)
         else:
             ops.attention_generic(q_lat, o_lat, cache.k, cache.v, ctx.token_req, ctx.positions, table, H, 1, C + R, s.softmax_scale,
                                   window=s.window, v_dim=C)
-        att = ops.latent_out(o_lat, self.uv_t, gate, H, C, E, out=take((n, H * E), x.dtype))
+        att = take((n, H * E), x.dtype)
+        if self._mfma_o:
+            ops.headwise_product(o_lat, C, self.uv, att, E, gate=gate)
+        else:
+            ops.latent_out(o_lat, self.uv, gate, H, C, E, out=att)
         return self.wo(att, out=out if out is not None else take((n, s.hidden), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)
 
 

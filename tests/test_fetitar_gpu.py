@@ -606,7 +606,7 @@ def step_context(lens, starts, tables, want=()):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-@pytest.mark.parametrize("H,D,R,E,Q,C,window", [(3, 24, 8, 40, 48, 56, 50), (1, 16, 2, 48, 16, 16, 7), (8, 16, 16, 16, 64, 32, 0), (2, 48, 32, 64, 96, 160, 120)])
+@pytest.mark.parametrize("H,D,R,E,Q,C,window", [(3, 24, 8, 40, 48, 56, 50), (1, 16, 2, 48, 16, 16, 7), (8, 16, 16, 16, 64, 32, 0), (2, 48, 32, 64, 96, 160, 120), (5, 64, 32, 48, 64, 96, 40)])
 def test_latent_attention_part_over_two_steps(dtype, H, D, R, E, Q, C, window):
     """The mixer alone over a paged cache: a prompt portion, then a second portion beside nothing else, then single tokens;
     against the plain mixer over the whole sequence."""
