@@ -62,7 +62,20 @@ __device__ __forceinline__ int wmin_i(int v) {
   return v;
 }
 
+// SHARE: the four waves of a workgroup are four heads of one key/value head over the same tokens and the same range of
+// keys (the host asks for it only with hp = 1 and a group that is a multiple of four, and pages of 8 tokens or more), so
+// each block of 32 keys is fetched once per workgroup, a quarter by each wave, and read from LDS by all four; the next
+// block's pieces are on their way in registers while this one is used.  Without it every wave fetches its own.
+constexpr int KROW = HD + 8;          // elements of a key's row in LDS (16 bytes of padding)
+constexpr int VROW = 32 + 8;          // elements of a channel's row in LDS
+constexpr int KPIECES = 32 * (HD / 8);  // 16-byte pieces of a block's keys
+constexpr int VPIECES = VD * 4;         // ... and of its values (a channel's 32 keys are four pieces)
+constexpr int KPT = (KPIECES + 255) / 256, VPT = (VPIECES + 255) / 256;  // pieces a thread fetches
+
+template <bool SHARE>
 __global__ __launch_bounds__(256) void attn_wide_kernel(WideParams a) {
+  __shared__ __align__(16) bf16_t lk[SHARE ? 32 * KROW : 8];
+  __shared__ __align__(16) bf16_t lv[SHARE ? VD * VROW : 8];
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int c = lane & 15, g = lane >> 4;
   const int G = a.heads / a.kv_heads;
@@ -148,41 +161,125 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(WideParams a) {
       pv[t] = table[kv2[t] >> psh];
     }
   };
-  if (kb0 < kb1) lookup(kb0);
+  if (!SHARE && kb0 < kb1) lookup(kb0);
+
+  // SHARE: the pieces of a block that this thread fetches for the workgroup, held in registers until the block before is
+  // done with.  A key outside the pages that hold [wlo, whi) is read from the nearest such page instead: it is masked anyway.
+  bf16x8 rk[KPT], rv[VPT];
+  constexpr int NP = PS >= 32 ? 1 : 32 / PS;  // pages that a block of 32 keys touches
+  auto fetch = [&](int kb) {
+    const int key_base = kb * 32, plo = wlo >> psh, phi = (whi - 1) >> psh;
+    int pg[NP];
+#pragma unroll
+    for (int j = 0; j < NP; ++j) pg[j] = table[min(max((key_base >> psh) + j, plo), phi)];
+    auto page_at = [&](int j) {
+      int page = pg[0];
+#pragma unroll
+      for (int jj = 1; jj < NP; ++jj)
+        if (j == jj) page = pg[jj];
+      return page;
+    };
+#pragma unroll
+    for (int r = 0; r < KPT; ++r) {
+      const int p = threadIdx.x + r * 256;
+      if (p < KPIECES) {
+        const int row = p / (HD / 8), col = p % (HD / 8);
+        const int page = page_at(PS >= 32 ? 0 : row >> psh), tok = (key_base + row) & pmask;
+        rk[r] = *reinterpret_cast<const bf16x8*>(a.k_cache + (size_t)page * k_page + (((size_t)kvh * HD) << psh) + (size_t)tok * HD + col * 8);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < VPT; ++r) {
+      const int p = threadIdx.x + r * 256;
+      if (p < VPIECES) {
+        const int ch = p >> 2, key0 = (p & 3) * 8;
+        const int page = page_at(PS >= 32 ? 0 : key0 >> psh), tok = (key_base + key0) & pmask;
+        rv[r] = *reinterpret_cast<const bf16x8*>(a.v_cache + (size_t)page * v_page + (((size_t)kvh * VD + ch) << psh) + tok);
+      }
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int r = 0; r < KPT; ++r) {
+      const int p = threadIdx.x + r * 256;
+      if (p < KPIECES) *reinterpret_cast<bf16x8*>(&lk[(p / (HD / 8)) * KROW + (p % (HD / 8)) * 8]) = rk[r];
+    }
+#pragma unroll
+    for (int r = 0; r < VPT; ++r) {
+      const int p = threadIdx.x + r * 256;
+      if (p < VPIECES) *reinterpret_cast<bf16x8*>(&lv[(p >> 2) * VROW + (p & 3) * 8]) = rv[r];
+    }
+  };
+  if constexpr (SHARE) {
+    if (kb0 < kb1) fetch(kb0);
+  }
 
   for (int kb = kb0; kb < kb1; ++kb) {
     const int key_base = kb * 32;
-    const bf16_t* krow[2] = {kbase + (size_t)pk[0] * k_page + (size_t)(kk[0] & pmask) * HD,
-                             kbase + (size_t)pk[1] * k_page + (size_t)(kk[1] & pmask) * HD};
-    const bf16_t* vrow[2] = {vbase + (size_t)pv[0] * v_page + (kv2[0] & pmask), vbase + (size_t)pv[1] * v_page + (kv2[1] & pmask)};
-    if (kb + 1 < kb1) lookup(kb + 1);
+    const bf16_t* krow[2];
+    const bf16_t* vrow[2];
+    if constexpr (SHARE) {
+      __syncthreads();  // every wave is done with the block before
+      stash();
+      __syncthreads();
+      if (kb + 1 < kb1) fetch(kb + 1);
+    } else {
+      krow[0] = kbase + (size_t)pk[0] * k_page + (size_t)(kk[0] & pmask) * HD;
+      krow[1] = kbase + (size_t)pk[1] * k_page + (size_t)(kk[1] & pmask) * HD;
+      vrow[0] = vbase + (size_t)pv[0] * v_page + (kv2[0] & pmask);
+      vrow[1] = vbase + (size_t)pv[1] * v_page + (kv2[1] & pmask);
+      if (kb + 1 < kb1) lookup(kb + 1);
+    }
+    // a block's operands, from LDS or straight from the pages
+    auto k_wide = [&](int t, int i) {
+      if constexpr (SHARE) return *reinterpret_cast<const bf16x8*>(&lk[(t * 16 + c) * KROW + i * 32 + g * 8]);
+      else return *reinterpret_cast<const bf16x8*>(krow[t] + i * 32);
+    };
+    auto k_narrow = [&](int t, int i) {
+      if constexpr (SHARE) return *reinterpret_cast<const s16x4*>(&lk[(t * 16 + c) * KROW + i * 16 + g * 4]);
+      else return *reinterpret_cast<const s16x4*>(krow[t] + i * 16);
+    };
+    auto v_at = [&](int t, int dt) {
+      if constexpr (SHARE) return *reinterpret_cast<const bf16x4*>(&lv[(dt * 16 + c) * VROW + t * 16 + g * 4]);
+      else return *reinterpret_cast<const bf16x4*>(vrow[t] + dt * v_step);
+    };
 
-    // scores: s[t][j] is key key_base + 16 t + 4 g + j of column c
+    // scores: s[t][j] is key key_base + 16 t + 4 g + j of column c; both 16-key tiles' rows are asked for before the first
+    // product, so that a block costs one trip to memory for its keys
     f32x4 s[2];
+    if (WIDE) {
+      bf16x8 kf[2][NQ];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-      if (WIDE) {
-        bf16x8 kf[NQ];
+      for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) kf[i] = *reinterpret_cast<const bf16x8*>(krow[t] + i * 32);
+        for (int i = 0; i < NQ; ++i) kf[t][i] = k_wide(t, i);
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[i], qw[i], acc, 0, 0, 0);
-      } else {
-        s16x4 kf[NQ];
+      for (int t = 0; t < 2; ++t) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int i = 0; i < NQ; ++i) kf[i] = *reinterpret_cast<const s16x4*>(krow[t] + i * 16);
-#pragma unroll
-        for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf[i], qn[i], acc, 0, 0, 0);
+        for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[t][i], qw[i], acc, 0, 0, 0);
+        s[t] = acc;
       }
-      s[t] = acc;
+    } else {
+      s16x4 kf[2][NQ];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) kf[t][i] = k_narrow(t, i);
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < NQ; ++i) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf[t][i], qn[i], acc, 0, 0, 0);
+        s[t] = acc;
+      }
     }
     // the first piece of the values is on its way while the soft-max runs
     bf16x4 vf[VPIECE][2];
 #pragma unroll
     for (int d = 0; d < VPIECE; ++d) {
-      vf[d][0] = *reinterpret_cast<const bf16x4*>(vrow[0] + d * v_step);
-      vf[d][1] = *reinterpret_cast<const bf16x4*>(vrow[1] + d * v_step);
+      vf[d][0] = v_at(0, d);
+      vf[d][1] = v_at(1, d);
     }
 
     // soft-max weights of the block, and the rescaling of what has been summed so far
@@ -237,8 +334,8 @@ __global__ __launch_bounds__(256) void attn_wide_kernel(WideParams a) {
 #pragma unroll
         for (int d = 0; d < VPIECE; ++d)
           if (d0 + VPIECE + d < DT) {
-            nx[d][0] = *reinterpret_cast<const bf16x4*>(vrow[0] + (d0 + VPIECE + d) * v_step);
-            nx[d][1] = *reinterpret_cast<const bf16x4*>(vrow[1] + (d0 + VPIECE + d) * v_step);
+            nx[d][0] = v_at(0, d0 + VPIECE + d);
+            nx[d][1] = v_at(1, d0 + VPIECE + d);
           }
       }
 #pragma unroll
@@ -313,12 +410,20 @@ __global__ __launch_bounds__(64) void attn_wide_reduce_kernel(bf16_t* __restrict
   float acc[PER];
 #pragma unroll
   for (int p = 0; p < PER; ++p) acc[p] = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float ws = __shfl(wgt, s, 64);
+  for (int s0 = 0; s0 < splits; s0 += 4) {  // four ranges' loads in flight at a time
+    float v[4][PER];
 #pragma unroll
-    for (int p = 0; p < PER; ++p) {
-      const int d = lane + p * 64;
-      if (d < VD) acc[p] += po[(size_t)s * VD + d] * ws;
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int p = 0; p < PER; ++p) {
+        const int d = lane + p * 64;
+        v[i][p] = (s0 + i < splits && d < VD) ? po[(size_t)(s0 + i) * VD + d] : 0.f;
+      }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float ws = __shfl(wgt, (s0 + i) & 63, 64);
+#pragma unroll
+      for (int p = 0; p < PER; ++p) acc[p] += v[i][p] * ws;
     }
   }
   const size_t col = (size_t)(info.z + ti) * heads + head;
@@ -356,7 +461,15 @@ extern "C" int ns_attn_wide(void* out, void* part_o, void* part_ml, const void* 
   const long items = (long)n_tiles * qt * splits * kv_heads * ((G + hp - 1) / hp);
   const long blocks = (items + 3) / 4;
   if (blocks > 0x7fffffffL || heads > 65535) return NS_ERR_BAD_ARG;
-  attn_wide_kernel<<<(unsigned)blocks, 256, 0, stream>>>(a);
+  // prompt portions of a group of a multiple of four heads: the four waves of a workgroup share each block of keys.
+  // (Measured with 32 heads over one key/value head, 2,048 tokens, windows of 1,024: keys of 64 and values of 64 channels
+  // 60 against 85 us; keys of 544 and values of 512 channels 780 against 460 us: with heads that wide a wave's sums,
+  // its queries and the pieces in flight leave no room, and one workgroup a compute unit waits at every barrier.)
+  constexpr bool SHARE_PAYS = HD + VD <= 512;
+  if (SHARE_PAYS && hp == 1 && G % 4 == 0 && PS >= 8 && qt > 1)
+    attn_wide_kernel<true><<<(unsigned)blocks, 256, 0, stream>>>(a);
+  else
+    attn_wide_kernel<false><<<(unsigned)blocks, 256, 0, stream>>>(a);
   const int st = ns_launch_status();
   if (st != NS_OK || splits == 1) return st;
   const int tile_tokens = qt * 16 / hp;

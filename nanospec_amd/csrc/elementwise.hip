@@ -577,8 +577,34 @@ __global__ void silu_mul_bias_kernel(T* __restrict__ out, const T* __restrict__ 
   }
 }
 
+template <typename T>
+__global__ void silu_mul_bias_vec_kernel(T* __restrict__ out, const T* __restrict__ gu, const T* __restrict__ bias, int inter, size_t total_vec) {
+  constexpr int V = 16 / sizeof(T);
+  typedef T vec_t __attribute__((ext_vector_type(V)));
+  const int ivec = inter / V;
+  for (size_t e = (size_t)blockIdx.x * blockDim.x + threadIdx.x; e < total_vec; e += (size_t)gridDim.x * blockDim.x) {
+    const size_t n = e / ivec;
+    const int i = (int)(e - n * ivec);
+    const vec_t g = reinterpret_cast<const vec_t*>(gu + n * 2 * inter)[i], u = reinterpret_cast<const vec_t*>(gu + n * 2 * inter + inter)[i];
+    const vec_t bg = reinterpret_cast<const vec_t*>(bias)[i], bu = reinterpret_cast<const vec_t*>(bias + inter)[i];
+    vec_t y;
+#pragma unroll
+    for (int k = 0; k < V; ++k) {
+      const float gf = to_f(g[k]) + to_f(bg[k]);
+      y[k] = from_f<T>(gf / (1.f + expf(-gf)) * (to_f(u[k]) + to_f(bu[k])));
+    }
+    reinterpret_cast<vec_t*>(out + n * inter)[i] = y;
+  }
+}
+
 extern "C" int ns_silu_mul_bias(void* out, const void* gu, const void* bias, int n_rows, int inter, int dtype, hipStream_t stream) {
   if (n_rows <= 0 || inter <= 0 || !bias) return NS_ERR_BAD_ARG;
+  if (dtype == NS_DTYPE_BF16 && inter % 8 == 0 && !(((uintptr_t)out | (uintptr_t)gu | (uintptr_t)bias) & 15)) {
+    const size_t tv = (size_t)n_rows * (inter / 8);
+    const int nb = (int)((tv + 255) / 256 < 16384 ? (tv + 255) / 256 : 16384);
+    silu_mul_bias_vec_kernel<bf16_t><<<nb, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)gu, (const bf16_t*)bias, inter, tv);
+    return ns_launch_status();
+  }
   const size_t total = (size_t)n_rows * inter;
   const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256 : 65536);
   if (dtype == NS_DTYPE_F32)
