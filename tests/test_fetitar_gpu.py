@@ -673,7 +673,7 @@ def test_gated_feed_forward_with_biases(dtype, rows):
 
 @pytest.mark.parametrize("HD,VD,page,H,G,window,slope", [(48, 32, 4, 4, 2, 37, 8.0), (96, 64, 16, 4, 1, 0, 8.0), (80, 48, 8, 3, 3, 20, 0.0),
                                                          (160, 128, 16, 24, 1, 100, 0.0), (288, 176, 16, 2, 1, 70, 2.0),
-                                                         (64, 48, 8, 8, 2, 50, 8.0), (96, 80, 32, 4, 1, 33, 0.0)])
+                                                         (64, 48, 8, 8, 2, 50, 8.0), (96, 80, 32, 4, 1, 33, 0.0), (32, 16, 4, 6, 2, 9, 8.0)])
 def test_two_size_matrix_core_attention(HD, VD, page, H, G, window, slope):
     """Keys and values of two sizes on the matrix cores: a prompt portion behind cached keys beside three single tokens of
     other requests, with the keys in one range and cut into ranges; against the plain rows."""
