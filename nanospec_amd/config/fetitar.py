@@ -1,7 +1,7 @@
 """The Fetitar decoder's configuration, read from its own config.json keys.
 
 A Fetitar model is a list of layers over a 32-bit residual stream, each with a norm before AND behind each sublayer
-(x <- x + norm_b(sublayer(norm(x))), norm weights stored around zero), a mixer and an optional gated feed-forward with
+(x <- x + norm_b(sublayer(norm(x))), norm weights kept as the factor minus one), a mixer and an optional gated feed-forward with
 biases.  Mixers: "attention" (grouped soft-max attention without rotation: biased projections, an RMS norm over the whole
 of q and of k, a bias by distance with one slope per head, a sliding window, values optionally mixed with the values of
 the first such layer) and "latent_attention" (queries through a normed latent, keys and values from one cached latent and

@@ -17,7 +17,7 @@ from typing import ClassVar
 
 @dataclass(frozen=True)
 class RMSNormSpec:
-    """y = w * x / sqrt(mean(x^2) + eps) over the last axis.  ``unit_offset``: the stored weight lies around zero and the
+    """y = w * x / sqrt(mean(x^2) + eps) over the last axis.  ``unit_offset``: the stored weight is the factor minus one: the
     factor is 1 + w, formed in 32-bit."""
 
     kind: ClassVar[str] = "rmsnorm"

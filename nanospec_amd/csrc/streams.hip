@@ -4,7 +4,7 @@
 //   read:   u = sum_s a[s] x_s;            h = w * u / sqrt(mean(u^2) + eps)      (h in the model's precision)
 //   write:  x_t <- sum_s M[s][t] x_s + c[t] y     for all t at once, from the old streams
 // S = 1 with a = M = 1 is the plain pre-norm residual x <- x + c y with its sum in 32-bit.
-// Two options on either side.  A norm's stored weight may lie around zero: the factor is then ``w_offset`` + w with
+// Two options on either side.  A norm's stored weight may be the factor minus one: the factor is then ``w_offset`` + w with
 // w_offset = 1, formed in 32-bit (0 leaves the weight as it is).  A sublayer's output may pass a bias and an RMS norm of
 // its own on its way into the streams (a block with norms on both sides of a sublayer):
 //   y' = (y + bias) / sqrt(mean((y + bias)^2) + eps_y) * (yw_offset + yw),   then the write with y' in place of y.

@@ -17,7 +17,7 @@ class RMSNorm:
     def __init__(self, spec, name: str) -> None:
         self.spec, self.name = spec, name
         self.weight: torch.Tensor | None = None
-        # a weight stored around zero: the factor is 1 + w, which the kernels form in 32-bit from the stored value (1 + w
+        # a weight kept as the factor minus one: the factor is 1 + w, which the kernels form in 32-bit from the stored value (1 + w
         # rounded to bfloat16 would lose most of w)
         self.offset = 1.0 if getattr(spec, "unit_offset", False) else 0.0
         if self.offset:
@@ -31,7 +31,7 @@ class RMSNorm:
 
     def forward(self, ctx, resid=None, x=None, rows=None, write_resid=False, out=None) -> torch.Tensor:
         if self.offset:
-            raise ops.KernelRefused("a norm whose weight is stored around zero reads a 32-bit stream (blocks of kind 'streams')")
+            raise ops.KernelRefused("a norm whose weight is kept as the factor minus one reads a 32-bit stream (blocks of kind 'streams')")
         return ops.rmsnorm(self.weight, self.spec.eps, resid=resid, x=x, rows=rows, write_resid=write_resid, out=out)
 
     def read_streams(self, ctx, streams: torch.Tensor, coeff: torch.Tensor, rows=None, out=None, sum_out=None, pending=None,

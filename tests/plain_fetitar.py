@@ -19,7 +19,7 @@ def rms(x: torch.Tensor, eps: float) -> torch.Tensor:
 
 
 def norm_one_plus(x, w, eps):
-    """RMS norm whose stored weight lies around zero: the factor is 1 + w."""
+    """RMS norm whose stored weight is the factor minus one: the factor is 1 + w."""
     return rms(x, eps) * (1.0 + w.to(F))
 
 

@@ -41,6 +41,8 @@ def latent_layer(heads, dim, rot, vdim, q_rank, kv_rank, scale, window, ff, base
 #    rotation, embedding scale absent, multipliers of the pair table that make many pairs collide.
 # R: many small heads, a single layer that says v_mix (a source without readers), a window longer than every request,
 #    no pair table.
+# S: sizes that the matrix-core kernels take in bfloat16 (keys and values of two sizes, the per-head products of the latent
+#    layers), groups of four heads (prompt portions share keys through LDS) and of three, windows that pass over decoded tokens.
 CONFIGS = {
     "P": dict(cfg={"architecture": "Fetitar", "vocab": 300, "width": 90, "norm": {"eps": 1e-5},
                    "embedding": {"scale": 3.0, "bigram": {"buckets": 53, "mul_prev": 31, "mul_cur": 5}},
@@ -61,6 +63,13 @@ CONFIGS = {
                               attn_layer(8, 8, 16, 32, 0.25, 500, 128, v_mix=True),
                               latent_layer(8, 8, 4, 24, 32, 96, 0.4, 30, 64)]},
               seed=5, page=4, lengths=(5, 31, 64, 100)),
+    "S": dict(cfg={"architecture": "Fetitar", "vocab": 160, "width": 96, "norm": {"eps": 1e-6},
+                   "embedding": {"scale": 5.0, "bigram": {"buckets": 101, "mul_prev": 17, "mul_cur": 3}},
+                   "layers": [latent_layer(4, 32, 16, 32, 64, 64, 0.15, 60, 160, base=1e5, scaling=(8.0, 128, 32.0, 1.0)),
+                              attn_layer(8, 2, 48, 32, 0.12, 45, 128, v_mix=True),
+                              latent_layer(2, 64, 32, 48, 32, 96, 0.1, 200, None, base=1e4),
+                              attn_layer(6, 2, 48, 32, 0.12, 70, 96, v_mix=True)]},
+              seed=6, page=16, lengths=(2, 40, 97, 180, 260)),
 }
 # matrices that random weights of the usual law leave so small that every soft-max is flat: drawn larger here
 SHARPEN = {"mix.uq": 6.0, "mix.uk": 6.0, "mix.dkv": 3.0, "mix.q.norm": 2.0, "mix.g": 20.0, "mix.q.b": 20.0, "mix.k.b": 20.0, "mix.v.b": 20.0,
@@ -406,7 +415,7 @@ def test_pair_embedding_remembers_the_last_token_between_steps(dtype, buckets, m
 @pytest.mark.parametrize("S,W", [(1, 64), (1, 90), (2, 96), (1, 2048), (1, 4100), (5, 30)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_norms_on_both_sides_of_a_sublayer(S, W, dtype):
-    """x <- x + norm_b(y + bias) in 32-bit and then the read through the next norm, both with weights stored around zero;
+    """x <- x + norm_b(y + bias) in 32-bit and then the read through the next norm, both with weights kept as the factor minus one;
     in one pass where the sizes allow it and in two kernels where not, for all rows and for chosen rows that are not kept."""
     from nanospec_amd.kernels import ops
 
