@@ -55,6 +55,8 @@ struct NormLink {
   float* ssq_out;       // [M][workgroups]
   int resid_stride;
   int act;              // EPI_ACT: which activation
+  const bf16_t* bias;   // [N] or null: added to the 32-bit sums before the epilogue's arithmetic (EPI_STORE, EPI_ACT and the
+  const bf16_t* bias2;  // gated ones, where ``bias`` is the gate's and ``bias2`` the up matrix's)
 };
 
 __device__ __forceinline__ bf16x8 load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
@@ -260,6 +262,8 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
         s *= rinv_s[m];
         u *= rinv_s[m];
       }
+      if (nl.bias) s += (float)nl.bias[n];
+      if (nl.bias2) u += (float)nl.bias2[n];
       out[(size_t)m * out_stride + n] = (OutT)(s / (1.f + expf(-s)) * u);
     }
     return;
@@ -273,11 +277,13 @@ __global__ __launch_bounds__(WAVES * 64) void gemm_tiled_kernel(OutT* __restrict
 #pragma unroll
     for (int wv = 0; wv < WAVES; ++wv) s += red[wv][mt][le];
     if (nl.ssq_in) s *= rinv_s[m];
+    if ((EPI == EPI_STORE || EPI == EPI_ACT || EPI == EPI_SILU_MUL) && nl.bias) s += (float)nl.bias[n];
     if (EPI == EPI_SILU_MUL) {
       float u = 0.f;
 #pragma unroll
       for (int wv = 0; wv < WAVES; ++wv) u += red[wv][MT + mt][le];
       if (nl.ssq_in) u *= rinv_s[m];
+      if (nl.bias2) u += (float)nl.bias2[n];
       s = s / (1.f + expf(-s)) * u;
     }
     if (EPI == EPI_ACT) {
@@ -344,12 +350,15 @@ static int tiled_dispatch(void* out, const void* x, const void* wt, const void* 
 // ssq_in (may be null): x holds rows that a norm's weight has scaled but its 1/rms has not; see NormLink.
 extern "C" int ns_gemm_tiled_bf16(void* out, const void* x, const void* wt, const void* wt2, int M, int N, int K,
                                   int x_stride, int out_stride, int epi, int out_f32, int waves, const float* ssq_in,
-                                  int parts_in, int norm_dim, float eps, int act, hipStream_t stream) {
+                                  int parts_in, int norm_dim, float eps, int act, const void* bias, const void* bias2,
+                                  hipStream_t stream) {
   if (epi != EPI_STORE && epi != EPI_SILU_MUL && epi != EPI_GATED_HALF && epi != EPI_ACT) return NS_ERR_BAD_ARG;
   if (epi == EPI_ACT && (act < 0 || act > 1)) return NS_ERR_BAD_ARG;
+  if (bias2 && epi != EPI_SILU_MUL && epi != EPI_GATED_HALF) return NS_ERR_BAD_ARG;
   RopeKvParams rk = {};
   NormLink nl = {};
   nl.act = act;
+  nl.bias = (const bf16_t*)bias; nl.bias2 = (const bf16_t*)bias2;
   nl.ssq_in = ssq_in; nl.parts_in = parts_in; nl.inv_dim = norm_dim > 0 ? 1.f / (float)norm_dim : 0.f; nl.eps = eps;
   return tiled_dispatch(out, x, wt, wt2, M, N, K, x_stride, out_stride, epi, out_f32, waves, rk, nl, stream);
 }

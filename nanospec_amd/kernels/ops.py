@@ -357,8 +357,10 @@ GATED_HALF_ROWS = 4  # up to this many rows the gated product runs half a row ti
 
 
 def linear_tiled(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight | None = None, out: torch.Tensor | None = None,
-                 out_f32: bool = False, waves: int = 0, halves: bool | None = None, act: str | None = None) -> torch.Tensor:
-    """bfloat16 x @ w.T for at most 64 rows from a tiled weight; with ``w2``: silu(x @ w.T) * (x @ w2.T).  ``x`` may be a
+                 out_f32: bool = False, waves: int = 0, halves: bool | None = None, act: str | None = None,
+                 bias: torch.Tensor | None = None, bias2: torch.Tensor | None = None) -> torch.Tensor:
+    """bfloat16 x @ w.T for at most 64 rows from a tiled weight; with ``w2``: silu(x @ w.T) * (x @ w2.T).  ``bias`` (and, with
+    ``w2``, ``bias2``): bfloat16 [N], added to the 32-bit sums before anything else happens to them.  ``x`` may be a
     ``PreNormed`` (at most 16 rows).  ``halves`` (with ``w2``, at most 16 rows): a workgroup takes 8 rows of each matrix
     instead of 16, which spreads a number of row tiles that is no multiple of the compute units evenly; None: by rows.
     ``act`` (one of ``ACTIVATIONS``, not with ``w2`` or 32-bit results): the activation of the result, which is rounded to
@@ -380,6 +382,11 @@ def linear_tiled(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight 
         raise KernelRefused("linear_tiled: out has the wrong shape or dtype")
     if w2 is not None and (w2.n != w.n or w2.k != w.k):
         raise KernelRefused("linear_tiled: w2 must match w")
+    for b in (bias, bias2):
+        if b is not None and (not b.is_cuda or b.shape != (w.n,) or b.dtype != torch.bfloat16 or not b.is_contiguous()):
+            raise KernelRefused(f"linear_tiled: a bias is bfloat16 [{w.n}]")
+    if bias2 is not None and w2 is None:
+        raise KernelRefused("linear_tiled: a second bias goes with a second matrix")
     if waves == 0:  # with more than 8 rows eight waves were never behind four at the shapes measured
         waves = 8 if w.k >= 8192 or ((w.n // 16 < 512 or m > 8) and w.k >= 2048) else 4
     if halves is None:  # (with 3 or 4 rows only where whole row tiles would not spread evenly over 256 compute units)
@@ -389,7 +396,7 @@ def linear_tiled(x: "torch.Tensor | PreNormed", w: TiledWeight, w2: TiledWeight 
                                            c_int(w.n), c_int(w.k), c_int(x.stride(0)), c_int(out.stride(0)),
                                            c_int(epi), c_int(1 if out_f32 else 0), c_int(waves),
                                            *_prenorm_args(pre, m, "linear_tiled"), c_int(ACTIVATIONS[act] if act is not None else 0),
-                                           _stream()),
+                                           _ptr(bias), _ptr(bias2), _stream()),
            "linear_tiled")
     return out
 

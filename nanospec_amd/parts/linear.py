@@ -207,18 +207,25 @@ class LinearWeight:
 
 
 class GatedWeights:
-    """Gate and up matrices of a gated feed-forward: silu(x @ Wg^T) * (x @ Wu^T) in one pass over x."""
+    """Gate and up matrices of a gated feed-forward: silu(x @ Wg^T) * (x @ Wu^T) in one pass over x.  ``bias`` = (gate's,
+    up's): silu(x @ Wg^T + bg) * (x @ Wu^T + bu); up to 16 rows add them in the streaming product's epilogue, more rows go
+    through the product of the stacked matrices and a kernel that adds the biases and applies the activation."""
 
-    def __init__(self, gate: torch.Tensor, up: torch.Tensor, keep_plain: bool = True) -> None:
+    def __init__(self, gate: torch.Tensor, up: torch.Tensor, keep_plain: bool = True, bias: tuple | None = None) -> None:
         self.inter, self.k = gate.shape
         self.dtype = gate.dtype
         fast = gate.dtype == torch.bfloat16 and self.k % 8 == 0
         self.tiled = (ops.TiledWeight(gate), ops.TiledWeight(up)) if fast else None
-        self.stacked = torch.cat([gate, up]) if (keep_plain or not fast) else None  # [2 I, K] for the two-kernel path
+        self.bias = None if bias is None else (bias[0].contiguous(), bias[1].contiguous())
+        self.bias_stacked = None if bias is None else torch.cat(self.bias).contiguous()
+        # [2 I, K] for the two-kernel path (which biased products of more than 16 rows always take)
+        self.stacked = torch.cat([gate, up]) if (keep_plain or not fast or bias is not None) else None
         self._stacked_t = self.stacked.t() if self.stacked is not None else None
+        # biased and bfloat16: more than 16 rows take the stacked matrix in plain rows to the library (no third copy is re-laid)
+        self._stacked_linear = LinearWeight(self.stacked, keep_plain=True, tiled=False) if (bias is not None and fast) else None
 
     def links_norms(self, rows: int) -> bool:
-        return self.tiled is not None and rows <= STREAM_ROWS
+        return self.bias is None and self.tiled is not None and rows <= STREAM_ROWS
 
     def _few_rows(self, x, m: int, out: torch.Tensor) -> torch.Tensor:
         """Up to 16 rows (plain or pre-normed).  From a few rows on, where the number of row tiles deals unevenly to the
@@ -227,6 +234,8 @@ class GatedWeights:
         at 16); where the tiles deal evenly it is not (1B shape, 512 tiles: 2% of a decode step behind)."""
         tiles, units = -(-self.inter // 16), ops.compute_units(out.device)
         uneven = -(-tiles // units) * units > 1.05 * tiles  # a tile of each matrix per workgroup leaves some units a round short
+        if self.bias is not None:
+            return ops.linear_tiled(x, self.tiled[0], w2=self.tiled[1], out=out, bias=self.bias[0], bias2=self.bias[1])
         if m > ops.GATED_HALF_ROWS and uneven and ops.wide_waves(self.inter, self.k, m, 1, 1, gated=True, units=units)[1]:
             return ops.linear_wide(x, self.tiled[0], w2=self.tiled[1], out=out, ksplit=1, nt=1)
         return ops.linear_tiled(x, self.tiled[0], w2=self.tiled[1], out=out)
@@ -240,6 +249,13 @@ class GatedWeights:
         fast = self.tiled is not None and ops.tiled_takes(x[:1], self.k)
         if fast and m <= STREAM_ROWS:
             return self._few_rows(x, m, out)
+        if self.bias is not None:
+            gu = ctx.arena.take((m, 2 * self.inter), x.dtype)
+            if self._stacked_linear is not None:
+                self._stacked_linear(x, out=gu, arena=ctx.arena, plain_copy=not ctx.captured)
+            else:
+                ops.linear_generic(x, self.stacked, out=gu)
+            return ops.silu_mul_bias(gu, self.bias_stacked, out=out)
         # (an inner size that the library does not take in one piece: the hand-written kernels at every number of rows)
         stacked = self.stacked if (self.k <= LIBRARY_MAX_K or not fast) else None
         if fast and stacked is None and self.k <= LIBRARY_MAX_K and m >= UNTILE_MIN_ROWS and not ctx.captured:

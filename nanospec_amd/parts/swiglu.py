@@ -1,7 +1,8 @@
 """The dense SwiGLU feed-forward: down(silu(gate(x)) * up(x)) (reference: model/llama.py:187-195).
 Gate and up matrices are stacked at load time so that one pass over the input serves both.  With biases
-(``SwiGLUSpec.bias``) gate and up are one product of the stacked matrix and a kernel that adds the biases and applies the
-activation; the down-projection's bias is added behind it, or left to the block (``out_bias``)."""
+(``SwiGLUSpec.bias``) gate and up add theirs in the streaming product's epilogue for up to 16 rows, and for more rows are one
+product of the stacked matrix and a kernel that adds the biases and applies the activation; the down-projection's bias is
+added behind it, or left to the block (``out_bias``)."""
 
 from __future__ import annotations
 
@@ -46,8 +47,7 @@ class SwiGLU:
         g, u, d = self._names
         to = lambda name: get(name).to(device=device, dtype=dtype)
         if self.biased:
-            self.gate_up = LinearWeight(torch.cat([to(g), to(u)]).contiguous(), keep_plain=plain)
-            self.gate_up_bias = torch.cat([to(g + s.bias_suffix), to(u + s.bias_suffix)]).contiguous()
+            self.gate_up = GatedWeights(to(g), to(u), keep_plain=plain, bias=(to(g + s.bias_suffix), to(u + s.bias_suffix)))
             self.out_bias = to(d + s.bias_suffix).contiguous()
         else:
             self.gate_up = GatedWeights(to(g), to(u), keep_plain=plain)
@@ -60,8 +60,7 @@ class SwiGLU:
     def forward(self, ctx, x, out: torch.Tensor | None = None, residual=None, add_out_bias: bool = True):
         if self.biased:
             n = x.shape[0]
-            gu = self.gate_up(x, out=ctx.arena.take((n, 2 * self.spec.intermediate), x.dtype), arena=ctx.arena, plain_copy=not ctx.captured)
-            act = ops.silu_mul_bias(gu, self.gate_up_bias, out=ctx.arena.take((n, self.spec.intermediate), x.dtype))
+            act = self.gate_up(ctx, x, out=ctx.arena.take((n, self.spec.intermediate), x.dtype))
             y = self.down(act, out=out if out is not None else ctx.arena.take((n, self.spec.hidden), x.dtype), arena=ctx.arena,
                           plain_copy=not ctx.captured)
             return ops.add_bias(y, self.out_bias) if add_out_bias else y
