@@ -163,7 +163,9 @@ def wide_attention(ctx, q, out, cache, table, heads: int, kv_heads: int, head_di
             hp *= 2
         waves = decode_tiles.shape[0] * kv_heads * -(-group // hp)
         longest = min(ctx.max_kv_len, window) if window else ctx.max_kv_len
-        splits = max(1, min(32, 4 * units // max(1, waves), -(-longest // WIDE_RANGE_KEYS)))
+        # (wide heads: a block of 32 keys is a long chain of loads and products already, so ranges go down to one block)
+        range_keys = WIDE_RANGE_KEYS // 2 if head_dim + v_dim > 512 else WIDE_RANGE_KEYS
+        splits = max(1, min(32, 4 * units // max(1, waves), -(-longest // range_keys)))
         ws = None
         if splits > 1:
             cols = decode_tiles.shape[0] * (16 // hp) * heads
